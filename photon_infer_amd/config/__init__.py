@@ -1,6 +1,7 @@
 from .base import ConfigReader, architecture_name, read_config_json
 from .dafidra import DafidraConfig
+from .dokanex import DokanexConfig
 from .llama import LlamaConfig, RopeScaling
 from .rorevik import RorevikConfig
 
-__all__ = ["ConfigReader", "architecture_name", "read_config_json", "LlamaConfig", "RopeScaling", "DafidraConfig", "RorevikConfig"]
+__all__ = ["ConfigReader", "architecture_name", "read_config_json", "LlamaConfig", "RopeScaling", "DafidraConfig", "RorevikConfig", "DokanexConfig"]

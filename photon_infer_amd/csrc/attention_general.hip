@@ -5,7 +5,9 @@
 // For the query at absolute position p (include/photon/ops/kernels/mha_kernel.hpp:174-230):
 //   s_t = scale * <q, K[t]>, t = lo..p;  P = exp(s - max s) / sum exp(s - max s);
 //   o = sum_t P_t V[t]
-// with lo = 0, or p - window + 1 when a window is given.  Causality is the loop bound.
+// with lo = 0, or p - window + 1 when a window is given, or the start of p's chunk,
+// floor(p / chunk) * chunk, when positions are cut into chunks that do not see one another
+// (both given: the later of the two).  Causality is the loop bound.
 // The softmax is exact: no constant is added to the denominator (the reference's paged
 // kernel adds 1e-6, src/ops/kernels/cuda/paged_attention.cu:71).
 //
@@ -35,7 +37,7 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
     const T* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ req_of_token, const int* __restrict__ positions, int nh, int nkv, int hd, int page_size,
     float scale, int window, long num_pages, float* __restrict__ part, int vd, const float* __restrict__ slopes,
-    const float* __restrict__ sinks, const float* __restrict__ gate, float softcap, float out_mult) {
+    const float* __restrict__ sinks, const float* __restrict__ gate, float softcap, float out_mult, int chunk) {
   __shared__ float qs[PI_MAX_HEAD_DIM];
   __shared__ float ps[PI_WAVE];
   __shared__ long voff[PI_WAVE];   // values are stored [page, kv_head, head_dim, slot]
@@ -46,7 +48,8 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
   const T* qr = q + t * q_stride + (long)h * hd;
   for (int d = lane; d < hd; d += PI_WAVE) qs[d] = to_float(qr[d]);
   const int p = positions[t];
-  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  if (chunk > 0 && (p / chunk) * chunk > lo) lo = (p / chunk) * chunk;
   const int* bt = block_table + (long)req_of_token[t] * table_width;
   float m = -INFINITY, l = 0.f;
   float acc[PI_MAX_HEAD_DIM / PI_WAVE] = {0.f, 0.f, 0.f, 0.f};
@@ -215,12 +218,13 @@ extern "C" int pi_paged_attention_general(void* out, long out_stride, const void
                                           const int* req_of_token, const int* positions, int T, int nh, int nkv, int hd,
                                           int page_size, float scale, int window, long num_pages, int splits, void* part,
                                           long part_elems, int vd, const float* slopes, const float* sinks, const float* gate,
-                                          float softcap, float out_mult, hipStream_t stream) {
+                                          float softcap, float out_mult, int chunk, hipStream_t stream) {
   PI_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention: heads %d must be a positive multiple of kv heads %d", nh, nkv);
   PI_REQUIRE(hd > 0 && hd <= PI_MAX_HEAD_DIM, "attention: head_dim %d must be at most %d", hd, PI_MAX_HEAD_DIM);
   PI_REQUIRE(page_size > 0 && table_width > 0 && num_pages > 0, "attention: bad cache geometry page_size=%d table_width=%d pages=%ld", page_size, table_width, num_pages);
   PI_REQUIRE(nh <= 65535, "attention: too many heads (%d)", nh);
   PI_REQUIRE(window >= 0, "attention: window must be >= 0, got %d", window);
+  PI_REQUIRE(chunk >= 0, "attention: chunk must be >= 0, got %d", chunk);
   PI_REQUIRE(splits >= 1 && splits <= 65535, "attention: bad number of key ranges %d", splits);
   if (vd <= 0) vd = hd;
   PI_REQUIRE(vd <= PI_MAX_HEAD_DIM, "attention: value width %d must be at most %d", vd, PI_MAX_HEAD_DIM);
@@ -230,11 +234,11 @@ extern "C" int pi_paged_attention_general(void* out, long out_stride, const void
   if (dtype == PI_F32)
     hipLaunchKernelGGL(paged_attention_general_kernel<float>, grid, block, 0, stream, (float*)out, out_stride, (const float*)q,
                        q_stride, (const float*)k_cache, (const float*)v_cache, block_table, table_width, req_of_token,
-                       positions, nh, nkv, hd, page_size, scale, window, num_pages, (float*)part, vd, slopes, sinks, gate, softcap, out_mult);
+                       positions, nh, nkv, hd, page_size, scale, window, num_pages, (float*)part, vd, slopes, sinks, gate, softcap, out_mult, chunk);
   else if (dtype == PI_BF16)
     hipLaunchKernelGGL(paged_attention_general_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out, out_stride,
                        (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width,
-                       req_of_token, positions, nh, nkv, hd, page_size, scale, window, num_pages, (float*)part, vd, slopes, sinks, gate, softcap, out_mult);
+                       req_of_token, positions, nh, nkv, hd, page_size, scale, window, num_pages, (float*)part, vd, slopes, sinks, gate, softcap, out_mult, chunk);
   else
     return pi_fail("attention: unsupported dtype %d", dtype);
   if (pi_check_launch("paged_attention_general")) return -1;

@@ -156,6 +156,27 @@ __device__ inline float block_sum(float v, float* scratch) {
   return total;
 }
 
+// Block-wide sums of two values at once (one trip through LDS for both); `scratch` holds 32 floats.
+__device__ inline void block_sum2(float& a, float& b, float* scratch) {
+  a = wave_sum(a);
+  b = wave_sum(b);
+  const int wave = threadIdx.x / PI_WAVE, lane = threadIdx.x % PI_WAVE;
+  const int nwaves = (blockDim.x + PI_WAVE - 1) / PI_WAVE;
+  __syncthreads();
+  if (lane == 0) {
+    scratch[wave] = a;
+    scratch[16 + wave] = b;
+  }
+  __syncthreads();
+  float ta = 0.f, tb = 0.f;
+  for (int w = 0; w < nwaves; ++w) {
+    ta += scratch[w];
+    tb += scratch[16 + w];
+  }
+  a = ta;
+  b = tb;
+}
+
 // ---- error channel: entry points return 0 or a negative code and leave a message
 inline thread_local char pi_error_message[1024] = {0};
 

@@ -5,11 +5,11 @@
 PI_DEFINE_MODULE(core)
 
 // ------------------------------------------------------------------ embedding
-// out[t, :] = float(table[ids[t], :]).  An id outside [0, V) fills the row with NaN:
+// out[t, :] = float(table[ids[t], :]) * scale.  An id outside [0, V) fills the row with NaN:
 // loud in every later result, and no access outside the table.
 template <typename TW>
 __global__ void embedding_kernel(float* __restrict__ out, const TW* __restrict__ table,
-                                 const int* __restrict__ ids, int D, int V) {
+                                 const int* __restrict__ ids, int D, int V, float scale) {
   const long t = blockIdx.x;
   const int id = ids[t];
   float* o = out + t * D;
@@ -18,21 +18,38 @@ __global__ void embedding_kernel(float* __restrict__ out, const TW* __restrict__
     return;
   }
   const TW* row = table + (long)id * D;
-  for (int i = threadIdx.x; i < D; i += blockDim.x) o[i] = to_float(row[i]);
+  if (scale == 1.0f) {
+    for (int i = threadIdx.x; i < D; i += blockDim.x) o[i] = to_float(row[i]);
+  } else {
+    for (int i = threadIdx.x; i < D; i += blockDim.x) o[i] = to_float(row[i]) * scale;
+  }
 }
 
 extern "C" int pi_embedding(float* out, const void* table, int table_dtype, const int* ids, int T, int D,
-                            int V, hipStream_t stream) {
+                            int V, float scale, hipStream_t stream) {
   PI_REQUIRE(T >= 0 && D > 0 && V > 0, "embedding: bad sizes T=%d D=%d V=%d", T, D, V);
   if (T == 0) return 0;
   const int threads = D >= 256 ? 256 : 64;
   if (table_dtype == PI_F32)
-    hipLaunchKernelGGL(embedding_kernel<float>, dim3(T), dim3(threads), 0, stream, out, (const float*)table, ids, D, V);
+    hipLaunchKernelGGL(embedding_kernel<float>, dim3(T), dim3(threads), 0, stream, out, (const float*)table, ids, D, V, scale);
   else if (table_dtype == PI_BF16)
-    hipLaunchKernelGGL(embedding_kernel<bf16_t>, dim3(T), dim3(threads), 0, stream, out, (const bf16_t*)table, ids, D, V);
+    hipLaunchKernelGGL(embedding_kernel<bf16_t>, dim3(T), dim3(threads), 0, stream, out, (const bf16_t*)table, ids, D, V, scale);
   else
     return pi_fail("embedding: unsupported table dtype %d", table_dtype);
   return pi_check_launch("embedding");
+}
+
+// x <- cap * tanh(x / cap) over n float32 numbers, in place (logits that are capped on the way out).
+__global__ void softcap_kernel(float* __restrict__ x, long n, float cap) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) x[i] = cap * tanhf(x[i] / cap);
+}
+
+extern "C" int pi_softcap(float* x, long n, float cap, hipStream_t stream) {
+  PI_REQUIRE(n >= 0 && cap > 0.f, "softcap: bad arguments n=%ld cap=%g", n, (double)cap);
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(softcap_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x, n, cap);
+  return pi_check_launch("softcap");
 }
 
 // out[t, :] = float(table[ids[t], :]) * scale + float(pos_table[positions[t], :]): an embedding that is
@@ -328,10 +345,11 @@ extern "C" int pi_clamped_glu(void* out, int out_dtype, const void* gu, int gu_d
 // Pair j is (x[j], x[j + R/2]) or, interleaved, (x[2j], x[2j+1]);
 // (a, b) <- (a cos - b sin, a sin + b cos) with cos / sin of the token's angle from the
 // step's table (rope_table_kernel below).  Dims >= R are copied.
-// table[t, j] = cos(angle), table[t, R/2 + j] = sin(angle), angle = float(pos[t]) * inv_freq[j]:
+// table[t, j] = mult * cos(angle), table[t, R/2 + j] = mult * sin(angle), angle = float(pos[t]) * inv_freq[j]:
 // float32 product, full-range sine and cosine.  Made once per step and read by every layer.
+// `mult` is 1 for a plain rotation; a scaled rotation may stretch every rotated pair by a constant.
 __global__ void rope_table_kernel(float* __restrict__ table, const int* __restrict__ positions,
-                                  const float* __restrict__ inv_freq, int T, int half) {
+                                  const float* __restrict__ inv_freq, int T, int half, float mult) {
   const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= (long)T * half) return;
   const long t = idx / half;
@@ -339,15 +357,15 @@ __global__ void rope_table_kernel(float* __restrict__ table, const int* __restri
   const float angle = (float)positions[t] * inv_freq[j];
   float s, c;
   sincosf(angle, &s, &c);
-  table[t * 2 * half + j] = c;
-  table[t * 2 * half + half + j] = s;
+  table[t * 2 * half + j] = mult == 1.0f ? c : c * mult;
+  table[t * 2 * half + half + j] = mult == 1.0f ? s : s * mult;
 }
 
-extern "C" int pi_rope_table(float* table, const int* positions, const float* inv_freq, int T, int half, hipStream_t stream) {
+extern "C" int pi_rope_table(float* table, const int* positions, const float* inv_freq, int T, int half, float mult, hipStream_t stream) {
   PI_REQUIRE(T >= 0 && half > 0 && table && positions && inv_freq, "rope_table: bad arguments T=%d half=%d", T, half);
   if (T == 0) return 0;
   const long total = (long)T * half;
-  hipLaunchKernelGGL(rope_table_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, table, positions, inv_freq, T, half);
+  hipLaunchKernelGGL(rope_table_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, table, positions, inv_freq, T, half, mult);
   return pi_check_launch("rope_table");
 }
 

@@ -50,27 +50,6 @@ __global__ __launch_bounds__(256) void branch_norm_add_kernel(float* __restrict_
   }
 }
 
-// Block-wide sums of two values at once (one trip through LDS for both); `scratch` holds 32 floats.
-__device__ inline void block_sum2(float& a, float& b, float* scratch) {
-  a = wave_sum(a);
-  b = wave_sum(b);
-  const int wave = threadIdx.x / PI_WAVE, lane = threadIdx.x % PI_WAVE;
-  const int nwaves = (blockDim.x + PI_WAVE - 1) / PI_WAVE;
-  __syncthreads();
-  if (lane == 0) {
-    scratch[wave] = a;
-    scratch[16 + wave] = b;
-  }
-  __syncthreads();
-  float ta = 0.f, tb = 0.f;
-  for (int w = 0; w < nwaves; ++w) {
-    ta += scratch[w];
-    tb += scratch[16 + w];
-  }
-  a = ta;
-  b = tb;
-}
-
 // The same for rows of whole 16-byte groups, at most VPT groups per thread: a thread keeps its
 // values in registers between the passes, both branches' sums of squares share one reduction,
 // and every access is 16 bytes wide.  Few rows (decode steps) are a matter of latency: as many
@@ -189,27 +168,30 @@ extern "C" int pi_cast_stream(void* out, int out_dtype, const float* x, long n, 
   return pi_check_launch("cast_stream");
 }
 
-// ---------------------------------------------------------------- queries and keys normalised whole, then into the cache
-// One block per token.  The projection row (float32) holds [q: nh*hd | k: nkv*hd | v: nkv*vd | gate: ng].
-//   q <- q / sqrt(mean over ALL nh*hd entries + eps) * wq, times the token's temperature
-//        1 + coef * ln(floor((p + 1) / every) + 1)           (coef 0: none)
-//   k <- k / sqrt(mean over all nkv*hd entries + eps) * wk   -> key pages [page, kv head, slot, hd]
-//   v                                                         -> value pages [page, kv head, vd, slot]
+// ---------------------------------------------------------------- queries and keys normalised, then into the cache
+// One block per token.  The projection row (float32) holds [q: nh*hd | k: nkv*hd | v: nkv*vd | gate: ng]
+// (without the k and v columns when has_kv is 0: a layer that reads another layer's keys and values).
+//   per_head 0:  q <- q / sqrt(mean over ALL nh*hd entries + eps) * wq     (wq / wk null: no norm of that projection)
+//                k <- k / sqrt(mean over all nkv*hd entries + eps) * wk
+//   per_head 1:  every head of q and of k divided by the root mean square of its own hd entries (+ eps inside the
+//                root), times wq / wk where they are given
+//   q times the token's temperature 1 + coef * ln(floor((p + 1) / every) + 1)           (coef 0: none)
+//   k -> key pages [page, kv head, slot, hd];   v -> value pages [page, kv head, vd, slot]
 //   gate <- 1 / (1 + exp(-gate))                              -> float32 [T, ng]
-// wq / wk null: no norm of that projection.  `part` (with `splits` planes of `part_stride` floats, rows of
-// proj_stride columns): the projection as the float32 pieces of a product split over k, instead of `proj`.
+// `part` (with `splits` planes of `part_stride` floats, rows of proj_stride columns): the projection as the float32
+// pieces of a product split over k, instead of `proj`.
 template <typename T>
 __global__ __launch_bounds__(1024) void qk_norm_kv_write_kernel(
     T* __restrict__ q_out, long q_stride, float* __restrict__ gate_out, const float* __restrict__ proj, long proj_stride,
     const float* __restrict__ wq, const float* __restrict__ wk, const int* __restrict__ positions, const int* __restrict__ req_of_token,
     float eps, float temp_coef, int temp_every, int nh, int nkv, int hd, int vd, int ng, T* __restrict__ k_cache,
     T* __restrict__ v_cache, const int* __restrict__ block_table, int table_width, int page_size, long num_pages,
-    const float* __restrict__ part, int splits, long part_stride) {
+    const float* __restrict__ part, int splits, long part_stride, int per_head, int has_kv) {
   __shared__ float scratch[32];
   extern __shared__ float staged[];              // the token's row, when it comes in pieces
   const long t = blockIdx.x;
   const float* row = proj + t * proj_stride;
-  const int QN = nh * hd, KN = nkv * hd, VN = nkv * vd;
+  const int QN = nh * hd, KN = has_kv ? nkv * hd : 0, VN = has_kv ? nkv * vd : 0;
   if (part) {
     // the projection is still split over k: its float32 pieces are added here, in split order, once per element
     for (int i = threadIdx.x; i < QN + KN + VN + ng; i += blockDim.x) staged[i] = split_sum(part, splits, part_stride, t * proj_stride + i);
@@ -217,30 +199,64 @@ __global__ __launch_bounds__(1024) void qk_norm_kv_write_kernel(
     row = staged;
   }
   const int p = positions[t];
-  float sq = 0.f, sk = 0.f;
-  for (int i = threadIdx.x; i < QN; i += blockDim.x) sq = fmaf(row[i], row[i], sq);
-  for (int i = threadIdx.x; i < KN; i += blockDim.x) sk = fmaf(row[QN + i], row[QN + i], sk);
-  block_sum2(sq, sk, scratch);                   // both sums of squares in one trip through LDS
-  const float rq = wq ? 1.0f / sqrtf(sq / QN + eps) : 1.0f;
-  const float rk = wk ? 1.0f / sqrtf(sk / KN + eps) : 1.0f;
   const float temp = temp_coef != 0.f ? 1.0f + temp_coef * logf((float)((p + 1) / temp_every) + 1.0f) : 1.0f;
   T* qr = q_out + t * q_stride;
-  for (int i = threadIdx.x; i < QN; i += blockDim.x) {
-    float v = row[i];
-    if (wq) v = v * rq * wq[i];
-    qr[i] = from_float<T>(v * temp);
-  }
   for (int i = threadIdx.x; i < ng; i += blockDim.x) gate_out[t * ng + i] = 1.0f / (1.0f + expf(-row[QN + KN + VN + i]));
-  if (!k_cache) return;
-  const int blk = p / page_size, slot = p % page_size;
-  const long page = blk < table_width ? block_table[(long)req_of_token[t] * table_width + blk] : -1;
-  if (page < 0 || page >= num_pages) return;      // no page for this position: nothing is written
-  for (int i = threadIdx.x; i < KN; i += blockDim.x) {
-    float v = row[QN + i];
-    if (wk) v = v * rk * wk[i];
-    const int g = i / hd, d = i % hd;
-    k_cache[((page * nkv + g) * page_size + slot) * hd + d] = from_float<T>(v);
+  long page = -1;
+  int slot = 0;
+  if (k_cache && has_kv) {
+    const int blk = p / page_size;
+    slot = p % page_size;
+    page = blk < table_width ? block_table[(long)req_of_token[t] * table_width + blk] : -1;
+    if (page >= num_pages) page = -1;              // no page for this position: nothing is written
   }
+  if (per_head) {
+    // a wave per head: query heads first, then key heads; the sum of squares runs over the head's own entries
+    const int wave = threadIdx.x / PI_WAVE, lane = threadIdx.x % PI_WAVE, nwaves = blockDim.x / PI_WAVE;
+    for (int u = wave; u < nh + (has_kv ? nkv : 0); u += nwaves) {
+      const bool is_q = u < nh;
+      const float* src = row + (is_q ? u * hd : QN + (u - nh) * hd);
+      float ss = 0.f;
+      for (int d = lane; d < hd; d += PI_WAVE) ss = fmaf(src[d], src[d], ss);
+      ss = wave_sum(ss);
+      const float r = 1.0f / sqrtf(ss / hd + eps);
+      if (is_q) {
+        for (int d = lane; d < hd; d += PI_WAVE) {
+          float v = src[d] * r;
+          if (wq) v *= wq[u * hd + d];
+          qr[u * hd + d] = from_float<T>(v * temp);
+        }
+      } else if (page >= 0) {
+        const int g = u - nh;
+        for (int d = lane; d < hd; d += PI_WAVE) {
+          float v = src[d] * r;
+          if (wk) v *= wk[g * hd + d];
+          k_cache[((page * nkv + g) * page_size + slot) * hd + d] = from_float<T>(v);
+        }
+      }
+    }
+  } else {
+    float sq = 0.f, sk = 0.f;
+    for (int i = threadIdx.x; i < QN; i += blockDim.x) sq = fmaf(row[i], row[i], sq);
+    for (int i = threadIdx.x; i < KN; i += blockDim.x) sk = fmaf(row[QN + i], row[QN + i], sk);
+    block_sum2(sq, sk, scratch);                   // both sums of squares in one trip through LDS
+    const float rq = wq ? 1.0f / sqrtf(sq / QN + eps) : 1.0f;
+    const float rk = wk && KN ? 1.0f / sqrtf(sk / KN + eps) : 1.0f;
+    for (int i = threadIdx.x; i < QN; i += blockDim.x) {
+      float v = row[i];
+      if (wq) v = v * rq * wq[i];
+      qr[i] = from_float<T>(v * temp);
+    }
+    if (page >= 0) {
+      for (int i = threadIdx.x; i < KN; i += blockDim.x) {
+        float v = row[QN + i];
+        if (wk) v = v * rk * wk[i];
+        const int g = i / hd, d = i % hd;
+        k_cache[((page * nkv + g) * page_size + slot) * hd + d] = from_float<T>(v);
+      }
+    }
+  }
+  if (page < 0) return;
   for (int i = threadIdx.x; i < VN; i += blockDim.x) {
     const int g = i / vd, d = i % vd;
     v_cache[((page * nkv + g) * vd + d) * page_size + slot] = from_float<T>(row[QN + KN + i]);
@@ -251,23 +267,25 @@ extern "C" int pi_qk_norm_kv_write(void* q_out, long q_stride, float* gate_out, 
                                    const float* wq, const float* wk, const int* positions, const int* req_of_token, float eps,
                                    float temp_coef, int temp_every, int T, int nh, int nkv, int hd, int vd, int ng,
                                    void* k_cache, void* v_cache, const int* block_table, int table_width, int page_size,
-                                   long num_pages, const float* part, int splits, long part_stride, hipStream_t stream) {
+                                   long num_pages, const float* part, int splits, long part_stride, int per_head, int has_kv,
+                                   hipStream_t stream) {
   PI_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && hd > 0 && vd > 0 && ng >= 0, "qk norm: bad sizes");
-  PI_REQUIRE(proj_stride >= (long)nh * hd + (long)nkv * (hd + vd) + ng, "qk norm: projection rows of %ld hold no q, k, v and gates", proj_stride);
+  const long row_floats = (long)nh * hd + (has_kv ? (long)nkv * (hd + vd) : 0) + ng;
+  PI_REQUIRE(proj_stride >= row_floats, "qk norm: projection rows of %ld hold no q, k, v and gates", proj_stride);
   PI_REQUIRE(temp_coef == 0.f || temp_every > 0, "qk norm: the temperature's period must be positive, got %d", temp_every);
-  PI_REQUIRE(!k_cache || (v_cache && block_table && req_of_token && table_width > 0 && page_size > 0 && num_pages > 0),
+  PI_REQUIRE(!k_cache || (has_kv && v_cache && block_table && req_of_token && table_width > 0 && page_size > 0 && num_pages > 0),
              "qk norm: bad cache geometry");
   PI_REQUIRE(ng == 0 || gate_out, "qk norm: gates without a place for them");
   PI_REQUIRE((proj != nullptr) != (part != nullptr), "qk norm: give the projection as a tensor or as pieces");
   PI_REQUIRE(!part || (splits >= 1 && part_stride >= (long)T * proj_stride), "qk norm: bad pieces (%d planes of %ld floats)", splits, part_stride);
-  const long row_floats = (long)nh * hd + (long)nkv * (hd + vd) + ng;
   PI_REQUIRE(!part || row_floats * 4 <= 60000, "qk norm: rows of %ld floats in pieces do not fit the staging memory", row_floats);
   const size_t lds = part ? (size_t)row_floats * sizeof(float) : 0;
   if (T == 0) return 0;
   const int threads = T <= 64 ? 1024 : 256;      // few tokens (decode steps): the row's passes are a matter of latency
 #define QKN_GO(TT) hipLaunchKernelGGL(qk_norm_kv_write_kernel<TT>, dim3(T), dim3(threads), lds, stream, (TT*)q_out, q_stride, gate_out, proj, \
                                       proj_stride, wq, wk, positions, req_of_token, eps, temp_coef, temp_every, nh, nkv, hd, vd, ng,  \
-                                      (TT*)k_cache, (TT*)v_cache, block_table, table_width, page_size, num_pages, part, splits, part_stride)
+                                      (TT*)k_cache, (TT*)v_cache, block_table, table_width, page_size, num_pages, part, splits, part_stride, \
+                                      per_head, has_kv)
   if (dtype == PI_F32) QKN_GO(float);
   else if (dtype == PI_BF16) QKN_GO(bf16_t);
   else return pi_fail("qk norm: unsupported dtype %d", dtype);

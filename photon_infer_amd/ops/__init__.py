@@ -100,7 +100,7 @@ def check_general_attention_sizes(num_heads: int, num_kv_heads: int, head_dim: i
 # ----------------------------------------------------------------------------- ops
 def embedding(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0,
               pos_table: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None) -> None:
-    """out[t, :] = float32(table[ids[t], :]); with a learned position table,
+    """out[t, :] = float32(table[ids[t], :]) * scale; with a learned position table,
     out[t, :] = table[ids[t], :] * scale + pos_table[positions[t], :]."""
     _gpu(out, table, ids, pos_table, positions)
     T, D = out.shape
@@ -116,10 +116,18 @@ def embedding(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, scale: 
         _lib.call("core", "pi_embedding_positions", out.data_ptr(), table.data_ptr(), pos_table.data_ptr(), _dt(table), ids.data_ptr(),
                   positions.data_ptr(), float(scale), T, D, table.shape[0], pos_table.shape[0], _stream())
         return
-    if scale != 1.0:
-        raise KernelError("embedding: a scale comes with a position table")
     _lib.call("core", "pi_embedding", out.data_ptr(), table.data_ptr(), _dt(table), ids.data_ptr(), T, D,
-              table.shape[0], _stream())
+              table.shape[0], float(scale), _stream())
+
+
+def softcap_(x: torch.Tensor, cap: float) -> None:
+    """x <- cap * tanh(x / cap), in place, float32."""
+    _gpu(x)
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise KernelError("softcap: expected a contiguous float32 tensor")
+    if not cap > 0.0:
+        raise KernelError(f"softcap: the cap must be positive, got {cap}")
+    _lib.call("core", "pi_softcap", x.data_ptr(), x.numel(), float(cap), _stream())
 
 
 def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float,
@@ -267,15 +275,16 @@ def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, hd: int
     return k_cache.shape[0]
 
 
-def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
-    """float32 [T, 2 * half]: cos then sin of float32(position) * inv_freq[j], for every token."""
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, magnitude: float = 1.0) -> torch.Tensor:
+    """float32 [T, 2 * half]: cos then sin of float32(position) * inv_freq[j], for every token, each
+    times ``magnitude`` (a scaled rotation that also stretches the rotated pairs)."""
     _gpu(positions, inv_freq)
     T, half = positions.shape[0], inv_freq.numel()
     _i32(positions, "positions")
     if inv_freq.dtype != torch.float32 or not inv_freq.is_contiguous():
         raise KernelError("rope: the frequency table must be contiguous float32")
     table = torch.empty((T, 2 * half), dtype=torch.float32, device=positions.device)
-    _lib.call("core", "pi_rope_table", table.data_ptr(), positions.data_ptr(), inv_freq.data_ptr(), T, half, _stream())
+    _lib.call("core", "pi_rope_table", table.data_ptr(), positions.data_ptr(), inv_freq.data_ptr(), T, half, float(magnitude), _stream())
     return table
 
 
@@ -415,7 +424,7 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
                     page_size: int, scale: float, window: int = 0, ws: Optional[KernelWorkspace] = None, *,
                     value_dim: Optional[int] = None, slopes: Optional[torch.Tensor] = None,
                     sinks: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
-                    softcap: float = 0.0, out_scale: float = 1.0) -> None:
+                    softcap: float = 0.0, out_scale: float = 1.0, chunk: int = 0) -> None:
     """Causal attention of every token of the step over its request's pages.
 
     ``ctx`` carries ``positions`` and ``req_of_token`` ([T] int32), the step's shape on the host
@@ -426,9 +435,13 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
     ``slopes`` (float32 [heads]: slope * distance is taken off a key's scaled score), ``sinks``
     (float32 [heads]: exp(sink) joins the softmax's denominator once), ``gate`` (float32
     [T, heads]: multiplies a head's output), ``softcap`` (c > 0: the scaled score s becomes c * tanh(s / c)),
-    ``out_scale`` (a factor on every output, applied in float32 before the one rounding).
+    ``out_scale`` (a factor on every output, applied in float32 before the one rounding), ``chunk`` (C > 0: positions
+    are cut into chunks of C, counted from 0, and a token sees the keys of its own chunk only).
     """
     _gpu(out, q, k_cache, v_cache, block_table, ctx.positions, ctx.req_of_token)
+    chunk = int(chunk or 0)
+    if chunk < 0:
+        raise KernelError(f"attention: a chunk must be positive, got {chunk}")
     T = q.shape[0]
     vd = head_dim if value_dim is None else int(value_dim)
     softcap, out_scale = float(softcap or 0.0), float(out_scale)
@@ -455,17 +468,18 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
         # the matrix-core kernels take heads whose values are as wide as their keys, options included
         from . import fast
         if fast.paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_kv_heads, head_dim,
-                                page_size, scale, window, pages, ws, slopes, sinks, gate, softcap, out_scale):
+                                page_size, scale, window, pages, ws, slopes, sinks, gate, softcap, out_scale, chunk):
             return
     # a step of few tokens over long contexts: its keys cut into ranges, merged by a second kernel
     # (as many as the context-length bucket asks for, so that a step gives the same bits eagerly and replayed)
-    ranges = general_attention_ranges(T, num_heads, int(ctx.max_kv_len))
+    # (chunks bound a token's keys whatever the context: one range)
+    ranges = general_attention_ranges(T, num_heads, min(int(ctx.max_kv_len), chunk) if chunk else int(ctx.max_kv_len))
     part = torch.empty(T * num_heads * ranges * (vd + 2), dtype=torch.float32, device=q.device) if ranges > 1 else None
     _lib.call("core", "pi_paged_attention_general", out.data_ptr(), _rows(out, "attention out"), q.data_ptr(),
               _rows(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(), _dt(q), block_table.data_ptr(),
               block_table.shape[1], ctx.req_of_token.data_ptr(), ctx.positions.data_ptr(), T, num_heads,
               num_kv_heads, head_dim, page_size, float(scale), int(window), pages, ranges, _ptr(part),
-              0 if part is None else part.numel(), vd, _ptr(slopes), _ptr(sinks), _ptr(gate), softcap, out_scale, _stream())
+              0 if part is None else part.numel(), vd, _ptr(slopes), _ptr(sinks), _ptr(gate), softcap, out_scale, chunk, _stream())
 
 
 def general_attention_ranges(tokens: int, num_heads: int, max_kv_len: int) -> int:
@@ -561,16 +575,22 @@ def branch_norm_add(x: torch.Tensor, a: torch.Tensor, w_outer: torch.Tensor, eps
 def qk_norm_kv_write(q_out: torch.Tensor, gate_out: Optional[torch.Tensor], proj: torch.Tensor, w_q: Optional[torch.Tensor],
                      w_k: Optional[torch.Tensor], ctx, eps: float, temp_coef: float, temp_every: int, num_heads: int,
                      num_kv_heads: int, head_dim: int, value_dim: int, num_gates: int, k_cache: Optional[torch.Tensor],
-                     v_cache: Optional[torch.Tensor], block_table: Optional[torch.Tensor], page_size: int) -> None:
+                     v_cache: Optional[torch.Tensor], block_table: Optional[torch.Tensor], page_size: int,
+                     per_head: bool = False, has_kv: bool = True) -> None:
     """From float32 projection rows [q | k | v | gates] (a tensor, or ``Partials``: the product still split over k,
     whose pieces are added here): queries and keys each normalised over their
     WHOLE row (all heads at once; weights float32, None: no norm), queries times the position's
     temperature 1 + coef * ln(floor((p + 1) / every) + 1), keys and values into their pages,
-    gates through a sigmoid into ``gate_out`` (float32 [T, num_gates])."""
+    gates through a sigmoid into ``gate_out`` (float32 [T, num_gates]).
+    ``per_head``: every head of q and k is divided by the root mean square of its own entries instead (weights, when
+    given, still multiply).  ``has_kv`` False: the rows hold [q | gates] only (keys and values are another layer's)."""
     pieces = proj if isinstance(proj, Partials) else None
     _gpu(q_out, gate_out, pieces.part if pieces is not None else proj, w_q, w_k, k_cache, v_cache, block_table)
     T = q_out.shape[0]
-    QN, KN, VN = num_heads * head_dim, num_kv_heads * head_dim, num_kv_heads * value_dim
+    QN = num_heads * head_dim
+    KN, VN = (num_kv_heads * head_dim, num_kv_heads * value_dim) if has_kv else (0, 0)
+    if not has_kv and k_cache is not None:
+        raise KernelError("qk norm: a cache to write without keys and values in the projection")
     if pieces is not None:
         if pieces.M != T or pieces.N < QN + KN + VN + num_gates:
             raise KernelError(f"qk norm: pieces [{pieces.M}, {pieces.N}] do not hold q, k, v and gates of {T} tokens")
@@ -579,7 +599,7 @@ def qk_norm_kv_write(q_out: torch.Tensor, gate_out: Optional[torch.Tensor], proj
     if q_out.shape[1] != QN:
         raise KernelError(f"qk norm: q has {q_out.shape[1]} columns, expected {QN}")
     _f32_vector(w_q, QN, "qk norm query weight")
-    _f32_vector(w_k, KN, "qk norm key weight")
+    _f32_vector(w_k if has_kv else None, KN, "qk norm key weight")
     if num_gates and (gate_out is None or gate_out.dtype != torch.float32 or not gate_out.is_contiguous() or gate_out.numel() != T * num_gates):
         raise KernelError(f"qk norm: gates need contiguous float32 [{T}, {num_gates}]")
     pages = 0
@@ -595,7 +615,81 @@ def qk_norm_kv_write(q_out: torch.Tensor, gate_out: Optional[torch.Tensor], proj
               float(temp_coef), int(temp_every), T, num_heads, num_kv_heads, head_dim, value_dim, num_gates, _ptr(k_cache),
               _ptr(v_cache), _ptr(block_table), block_table.shape[1] if k_cache is not None else 0, page_size, pages,
               pieces.part.data_ptr() if pieces is not None else None, pieces.splits if pieces is not None else 0,
+              pieces.M * pieces.N if pieces is not None else 0, int(bool(per_head)), int(bool(has_kv)), _stream())
+
+
+# ----------------------------------------------------------------------------- attention through a latent
+def latent_kv_write(cq_out: Optional[torch.Tensor], proj, w_q: Optional[torch.Tensor], w_kv: torch.Tensor, table: Optional[torch.Tensor],
+                    ctx, eps: float, q_rank: int, kv_rank: int, rot: int, k_cache: Optional[torch.Tensor],
+                    v_cache: Optional[torch.Tensor], block_table: Optional[torch.Tensor], page_size: int) -> None:
+    """From float32 projection rows [query latent: q_rank | key/value latent: kv_rank | shared rotated key part: rot]
+    (a tensor, or ``Partials``): the query latent RMS-normalised with ``w_q`` into ``cq_out`` ([T, q_rank], the
+    activation type); the key/value latent RMS-normalised with ``w_kv`` and the rotated part turned by the token's
+    angles (``table``: the step's [T, rot] cosines and sines, neighbouring pairs) into the pages: keys
+    [pages, 1, page, kv_rank + rot] = [latent | rotated part], values transposed [pages, 1, kv_rank (+ rot), page]."""
+    pieces = proj if isinstance(proj, Partials) else None
+    _gpu(cq_out, pieces.part if pieces is not None else proj, w_q, w_kv, table, k_cache, v_cache, block_table)
+    N = q_rank + kv_rank + rot
+    if pieces is not None:
+        T = pieces.M
+        if pieces.N < N:
+            raise KernelError(f"latent: pieces [{pieces.M}, {pieces.N}] do not hold {N} columns")
+    else:
+        T = proj.shape[0]
+        if proj.dtype != torch.float32 or proj.dim() != 2 or proj.shape[1] < N:
+            raise KernelError(f"latent: projection must be float32 [{T}, >= {N}], got {proj.dtype} {tuple(proj.shape)}")
+    if q_rank and (cq_out is None or cq_out.shape != (T, q_rank)):
+        raise KernelError(f"latent: the query latent's place must be [{T}, {q_rank}]")
+    _f32_vector(w_q, q_rank, "latent query norm weight")
+    _f32_vector(w_kv, kv_rank, "latent key norm weight")
+    if rot and (table is None or table.shape != (T, rot) or table.dtype != torch.float32 or not table.is_contiguous()):
+        raise KernelError(f"latent: cos / sin table must be contiguous float32 [{T}, {rot}]")
+    pages, v_rows = 0, kv_rank
+    dtype = cq_out.dtype if cq_out is not None else (k_cache.dtype if k_cache is not None else torch.float32)
+    if k_cache is not None:
+        v_rows = v_cache.shape[2] if v_cache.dim() == 4 else -1
+        if v_rows not in (kv_rank, kv_rank + rot):
+            raise KernelError(f"latent: values of {v_rows} rows are neither the latent's {kv_rank} nor the key's {kv_rank + rot}")
+        pages = _check_cache(k_cache, v_cache, 1, kv_rank + rot, page_size, dtype, v_rows)
+        if block_table.dim() != 2 or block_table.dtype != torch.int32 or not block_table.is_contiguous():
+            raise KernelError("latent: block table must be contiguous int32 [requests, width]")
+    _i32(ctx.positions, "positions", T)
+    _i32(ctx.req_of_token, "req_of_token", T)
+    _lib.call("core", "pi_latent_kv_write", _ptr(cq_out), _rows(cq_out, "query latent") if cq_out is not None else 0,
+              PI_F32 if dtype == torch.float32 else PI_BF16, None if pieces is not None else proj.data_ptr(),
+              pieces.N if pieces is not None else _rows(proj, "projection"), _ptr(w_q), w_kv.data_ptr(), _ptr(table),
+              ctx.positions.data_ptr(), ctx.req_of_token.data_ptr(), float(eps), T, q_rank, kv_rank, rot, v_rows, _ptr(k_cache),
+              _ptr(v_cache), _ptr(block_table), block_table.shape[1] if k_cache is not None else 0, page_size, pages,
+              pieces.part.data_ptr() if pieces is not None else None, pieces.splits if pieces is not None else 0,
               pieces.M * pieces.N if pieces is not None else 0, _stream())
+
+
+def head_gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, heads: int, a_head: Optional[int] = None,
+              out_head: Optional[int] = None, rot: int = 0, table: Optional[torch.Tensor] = None) -> None:
+    """A product per head: ``out[t, h * out_head + n] = sum_k a[t, h * a_head + k] * w[h, k, n]`` with ``w``
+    [heads, K, N] (a head's matrix stored with its inputs as rows), float32 sums.  ``a_head`` / ``out_head``: the
+    distance between two heads in a row of ``a`` / ``out`` (default K + rot / N + rot).  ``rot`` > 0: the ``rot`` numbers
+    behind a head's K inputs are turned by the token's angles (``table``: the step's [T, rot] cosines and sines,
+    neighbouring pairs) and placed behind the head's N results."""
+    _gpu(out, a, w, table)
+    if w.dim() != 3 or w.shape[0] != heads or not w.is_contiguous():
+        raise KernelError(f"head product: weights must be contiguous [{heads}, K, N], got {tuple(w.shape)}")
+    K, N = int(w.shape[1]), int(w.shape[2])
+    a_head = K + rot if a_head is None else int(a_head)
+    out_head = N + rot if out_head is None else int(out_head)
+    M = a.shape[0]
+    if a.dim() != 2 or out.dim() != 2 or out.shape[0] != M or a.dtype != out.dtype or w.dtype != a.dtype:
+        raise KernelError(f"head product: a {tuple(a.shape)} {a.dtype}, w {w.dtype}, out {tuple(out.shape)} {out.dtype} do not agree")
+    if a.shape[1] < (heads - 1) * a_head + K + rot or out.shape[1] < (heads - 1) * out_head + N + rot:
+        raise KernelError(f"head product: rows of {a.shape[1]} / {out.shape[1]} numbers do not hold {heads} heads of {a_head} / {out_head}")
+    if rot and (table is None or table.shape != (M, rot) or table.dtype != torch.float32 or not table.is_contiguous()):
+        raise KernelError(f"head product: cos / sin table must be contiguous float32 [{M}, {rot}]")
+    if _FAST and a.dtype == torch.bfloat16 and rot == 0:
+        from . import fast
+        if fast.head_gemm(out, a, w, heads, K, N, a_head, out_head):
+            return
+    _lib.call("core", "pi_head_gemm", out.data_ptr(), _rows(out, "head product out"), out_head, a.data_ptr(), _rows(a, "head product a"),
+              a_head, w.data_ptr(), _dt(a), M, heads, K, N, int(rot), _ptr(table), _stream())
 
 
 # ----------------------------------------------------------------------------- matrix memory

@@ -15,7 +15,8 @@ P, I, L, F = c_void_p, c_int, c_long, c_float
 # entry point -> argument types (all return int: 0 = ok)
 _SIGNATURES = {
     "core": {
-        "pi_embedding": [P, P, I, P, I, I, I, P],
+        "pi_embedding": [P, P, I, P, I, I, I, F, P],
+        "pi_softcap": [P, L, F, P],
         "pi_embedding_positions": [P, P, P, I, P, P, F, I, I, I, I, P],
         "pi_clamped_glu": [P, I, P, I, P, P, P, I, F, F, I, I, P, I, I, P],
         "pi_causal_conv_silu": [P, L, P, L, P, P, I, I, I, P, P, I, I, P, L, P],
@@ -26,10 +27,12 @@ _SIGNATURES = {
         "pi_swiglu": [P, P, I, I, I, I, P],
         "pi_rope_kv_write": [P, L, P, L, P, L, I, P, P, P, I, I, I, I, I, I, I, P, P, P, I, I, L, P, I, I, I, I, I, I, P],
         "pi_gemm_general": [P, I, L, P, I, L, P, I, L, I, I, I, I, P],
-        "pi_paged_attention_general": [P, L, P, L, P, P, I, P, I, P, P, I, I, I, I, I, F, I, L, I, P, L, I, P, P, P, F, F, P],
+        "pi_paged_attention_general": [P, L, P, L, P, P, I, P, I, P, P, I, I, I, I, I, F, I, L, I, P, L, I, P, P, P, F, F, I, P],
         "pi_branch_norm_add": [P, P, I, P, P, P, P, P, F, F, I, I, P],
         "pi_cast_stream": [P, I, P, L, P],
-        "pi_qk_norm_kv_write": [P, L, P, I, P, L, P, P, P, P, F, F, I, I, I, I, I, I, I, P, P, P, I, I, L, P, I, L, P],
+        "pi_qk_norm_kv_write": [P, L, P, I, P, L, P, P, P, P, F, F, I, I, I, I, I, I, I, P, P, P, I, I, L, P, I, L, I, I, P],
+        "pi_latent_kv_write": [P, L, I, P, L, P, P, P, P, P, F, I, I, I, I, I, P, P, P, I, I, L, P, I, L, P],
+        "pi_head_gemm": [P, L, I, P, L, I, P, I, I, I, I, I, I, P, P],
         "pi_matrix_memory_scan": [P, L, P, L, I, I, I, I, I, P, P, F, F, P, P, I, P, L, I, I, I, I, I, I, P, L, P],
         "pi_head_norm_gate": [P, I, P, L, P, L, P, F, I, I, I, F, P],
         "pi_route": [P, P, P, L, I, I, I, I, I, I, P],
@@ -38,7 +41,7 @@ _SIGNATURES = {
         "pi_grouped_gemm_general": [P, I, L, P, I, L, P, I, L, L, P, P, P, I, I, I, P],
         "pi_combine_choices": [P, P, P, P, I, I, I, I, P],
         "pi_paged_attention_general_ranges": [I, I, I],
-        "pi_rope_table": [P, P, P, I, I, P],
+        "pi_rope_table": [P, P, P, I, I, F, P],
         "pi_sample": [P, P, L, P, P, I, I, P, L, P],
         "pi_sample_static": [P, P, L, P, P, I, I, P],
     },

@@ -27,7 +27,7 @@ CSRC_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__
 # matrix-core kernels that only the bfloat16 path uses.
 MODULES: Dict[str, List[str]] = {
     "core": ["elementwise.hip", "gemm_general.hip", "attention_general.hip", "sampling.hip", "stream_norm.hip",
-             "matrix_memory.hip", "routed_experts.hip", "recurrent.hip"],
+             "matrix_memory.hip", "routed_experts.hip", "recurrent.hip", "latent.hip"],
     "bf16": ["gemm_mfma.hip", "gemm_skinny.hip", "attention_mfma.hip", "attention_decode.hip"],
     # host only: cache manager bookkeeping (needs no GPU and no hipcc)
     "runtime": ["runtime/cache.cpp"],

@@ -303,6 +303,11 @@ def gemm_clamped_glu(out, a, w, bias, limit, alpha, M, N, K, lda, ldw) -> bool:
     return True
 
 
+def head_gemm(out, a, w, heads: int, K: int, N: int, a_head: int, out_head: int) -> bool:
+    """A product per head on the matrix-core kernels; False: not for these sizes."""
+    return False
+
+
 # ----------------------------------------------------------------------------- attention
 def attention_tile_rows(num_heads: int, num_kv_heads: int, head_dim: int) -> int:
     return _lib.load("bf16").pi_attention_tile_rows(num_heads, num_kv_heads, head_dim)
@@ -511,11 +516,13 @@ def _decode_splits_that_fit(ws, n_req: int, num_heads: int, num_kv_heads: int, h
 
 def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_kv_heads, head_dim,
                     page_size, scale, window, pages, ws: Optional[KernelWorkspace] = None, slopes=None, sinks=None, gate=None,
-                    softcap: float = 0.0, out_scale: float = 1.0) -> bool:
+                    softcap: float = 0.0, out_scale: float = 1.0, chunk: int = 0) -> bool:
     """``slopes`` / ``sinks`` (float32 [heads]) and ``gate`` (float32 [tokens, heads]): a distance bias, a sink in
     the softmax and an output gate per head (None: none); ``softcap`` > 0: scaled scores s become
     softcap * tanh(s / softcap); ``out_scale``: a factor on every output."""
     opt = tuple(None if t is None else t.data_ptr() for t in (slopes, sinks, gate)) + (float(softcap), float(out_scale))
+    if chunk:
+        return False
     if head_dim not in DECODE_HEAD_DIMS or page_size % 16 or q.data_ptr() % 16 or q.stride(0) % 8 or out.stride(0) % 4:
         return False
     G = num_heads // num_kv_heads

@@ -6,6 +6,7 @@ from .norm import RMSNorm
 from .rope import RotaryEmbedding, rope_frequencies
 from .attention import PagedAttention
 from .sink_attention import SinkWindowAttention
+from .latent_attention import LatentAttention
 from .matrix_memory import MatrixMemory
 from .state_space import StateSpaceMixer
 from .delta_rule import ChannelDeltaRule
@@ -20,5 +21,5 @@ __all__ = [
     "KVCacheSpec", "LayerCache", "Mixer", "Norm", "PAGE", "PagedCacheSpec", "PagedTensor", "Part", "PositionEncoding", "StateSpec",
     "StepContext", "RMSNorm", "RotaryEmbedding", "rope_frequencies", "PagedAttention", "SwiGLU",
     "PreNormBlock", "OutputNormBlock", "SinkWindowAttention", "MatrixMemory", "RoutedExperts", "LMHead", "TokenEmbedding", "CachePlan", "DecoderModel", "ModelSpec",
-    "RunEntry", "plan_cache", "StateSpaceMixer", "ChannelDeltaRule", "ClampedGLU", "SideBySide", "PositionedEmbedding",
+    "RunEntry", "plan_cache", "StateSpaceMixer", "ChannelDeltaRule", "ClampedGLU", "SideBySide", "PositionedEmbedding", "LatentAttention",
 ]

@@ -19,10 +19,11 @@ from .base import Part
 class TokenEmbedding(Part):
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, tensor_name: str = "weight"):
+    def __init__(self, vocab_size: int, hidden_size: int, tensor_name: str = "weight", scale: float = 1.0):
         self.vocab_size = int(vocab_size)
         self.hidden_size = int(hidden_size)
         self.tensor_name = tensor_name          # after the part's prefix; may be empty
+        self.scale = float(scale)               # a factor on every row as it enters the stream (the table itself stays as stored)
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
@@ -36,7 +37,7 @@ class TokenEmbedding(Part):
         """int32 [T] -> float32 residual stream [T, hidden].  ``ctx``: the step's context, for
         embeddings that look at more than the ids."""
         x = torch.empty((token_ids.shape[0], self.hidden_size), dtype=torch.float32, device=token_ids.device)
-        ops.embedding(x, self.weight, token_ids)
+        ops.embedding(x, self.weight, token_ids, self.scale)
         return x
 
 
@@ -47,8 +48,8 @@ class PositionedEmbedding(TokenEmbedding):
 
     def __init__(self, vocab_size: int, hidden_size: int, max_positions: int, scale: float = 1.0, norm=None,
                  tensor_name: str = "weight", position_name: str = "positions"):
-        super().__init__(vocab_size, hidden_size, tensor_name)
-        self.max_positions, self.scale = int(max_positions), float(scale)
+        super().__init__(vocab_size, hidden_size, tensor_name, scale)
+        self.max_positions = int(max_positions)
         self.position_name = position_name
         self.norm_prefix, self.norm = norm if norm is not None else ("", None)
 
@@ -78,10 +79,11 @@ class PositionedEmbedding(TokenEmbedding):
 class LMHead(Part):
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, tied: bool, tensor_name: str = "weight"):
+    def __init__(self, vocab_size: int, hidden_size: int, tied: bool, tensor_name: str = "weight", softcap: Optional[float] = None):
         self.vocab_size = int(vocab_size)
         self.hidden_size = int(hidden_size)
         self.tied = bool(tied)
+        self.softcap = float(softcap) if softcap else 0.0     # c > 0: logits become c * tanh(logits / c)
         self.tensor_name = tensor_name          # after the part's prefix; may be empty
         self.weight: Optional[torch.Tensor] = None
 
@@ -99,4 +101,6 @@ class LMHead(Part):
         """activations [M, hidden] -> float32 logits [M, vocab]."""
         logits = torch.empty((h.shape[0], self.vocab_size), dtype=torch.float32, device=h.device)
         ops.gemm(logits, h, self.weight, ws=ctx.workspace if ctx is not None else None)
+        if self.softcap > 0.0:
+            ops.softcap_(logits, self.softcap)
         return logits

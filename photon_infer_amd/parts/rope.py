@@ -20,8 +20,25 @@ from typing import Optional
 
 import torch
 
+from dataclasses import dataclass
+
 from ..errors import UnsupportedModelError
 from .base import POSITION_ENCODINGS, PositionEncoding
+
+
+@dataclass(frozen=True)
+class RampScaling:
+    """Frequencies blended from f to f / factor by a ramp over the pair index (see the module's text)."""
+
+    factor: float
+    original: float        # the length the unscaled rotation was meant for
+    fast: float            # turns within that length from which on a pair keeps its frequency
+    slow: float            # turns within that length up to which a pair is slowed by the whole factor
+    rope_type: str = "ramp"
+
+    @property
+    def magnitude(self) -> float:
+        return 0.1 * math.log(self.factor) + 1.0
 
 
 def rope_frequencies(rotary_dim: int, theta: float, scaling=None) -> torch.Tensor:
@@ -42,6 +59,13 @@ def rope_frequencies(rotary_dim: int, theta: float, scaling=None) -> torch.Tenso
         out = torch.where(wavelen > L / lo, freq / factor, freq)
         is_mid = (wavelen <= L / lo) & (wavelen >= L / hi)
         return torch.where(is_mid, mid, out)
+    if scaling.rope_type == "ramp":
+        R, base = float(rotary_dim), float(theta)
+        where = lambda turns: R * math.log(float(scaling.original) / (2.0 * math.pi * float(turns))) / (2.0 * math.log(base))
+        lo = max(math.floor(where(scaling.fast)), 0)
+        hi = min(math.ceil(where(scaling.slow)), rotary_dim - 1)
+        ramp = torch.clamp((j - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        return freq / float(scaling.factor) * ramp + freq * (1.0 - ramp)
     raise UnsupportedModelError(f"rope scaling '{scaling.rope_type}' is not supported")
 
 
@@ -59,6 +83,8 @@ class RotaryEmbedding(PositionEncoding):
         self.theta = float(theta)
         self.scaling = scaling
         self.interleaved = bool(interleaved)
+        # a factor on every cosine and sine (1 unless the scaling rule stretches the rotated pairs)
+        self.magnitude = float(getattr(scaling, "magnitude", 1.0)) if scaling is not None else 1.0
         self.inv_freq: Optional[torch.Tensor] = None
 
     def load(self, tensors, dtype, device) -> None:
@@ -73,11 +99,13 @@ class RotaryEmbedding(PositionEncoding):
         cos / sin table instead of the frequencies: every layer of a step rotates by the same
         angles, so they are computed once."""
         if ctx is None:
+            if self.magnitude != 1.0:
+                raise UnsupportedModelError("a rotation that stretches its pairs is given by a step's table, not by its frequencies")
             return self.inv_freq, self.rotary_dim, self.interleaved
         table = ctx.scratch.get(("rope", id(self)))
         if table is None:
             from .. import ops
-            table = ctx.scratch[("rope", id(self))] = ops.rope_table(ctx.positions, self.inv_freq)
+            table = ctx.scratch[("rope", id(self))] = ops.rope_table(ctx.positions, self.inv_freq, self.magnitude)
         return table, self.rotary_dim, self.interleaved
 
 
