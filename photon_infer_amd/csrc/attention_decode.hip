@@ -7,7 +7,7 @@
 // the result is written directly.
 //
 // For the query at position p = kv_len - 1: keys lo..p with lo = max(0, p - window + 1)
-// (window 0: all keys).  Ranges are cut at multiples of 32 keys.
+// (window 0: all keys), or the start of p's chunk where positions are cut into chunks.  Ranges are cut at multiples of 32 keys.
 //
 // FUSED: the kernel starts from the q|k|v projection as the product left it (a bfloat16 tensor
 // or float32 pieces split over k) instead of rotated queries and a written cache: every wave
@@ -185,7 +185,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 2
   const int G = nh / nkv;
   const int kv_len = kv_len_of[r];
   const int p = kv_len - 1;
-  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const int lo = first_seen_key(p, window, opt.chunk);
   const long row = q_start[r];
   const int* bt = block_table + (long)r * table_width;
 
@@ -425,10 +425,11 @@ extern "C" int pi_attention_decode(void* out, long out_stride, const void* q, lo
                                    const int* kv_len, const int* req_ids, int R, int nh, int nkv, int hd, int page_size,
                                    float scale, int window, long num_pages, int splits, void* part, long part_elems,
                                    const float* slopes, const float* sinks, const float* gate, float softcap, float out_mult,
-                                   hipStream_t stream) {
+                                   int chunk, hipStream_t stream) {
+  PI_REQUIRE(chunk >= 0, "attention_decode: chunk must be >= 0, got %d", chunk);
   return launch_decode(false, DecodeSource{}, out, out_stride, q, q_stride, k_cache, v_cache, block_table, table_width, q_start,
                        kv_len, req_ids, R, nh, nkv, hd, page_size, scale, window, num_pages, splits, part, part_elems, true, stream,
-                       AttnOptions{slopes, sinks, gate, softcap, out_mult});
+                       AttnOptions{slopes, sinks, gate, softcap, out_mult, chunk});
 }
 
 // The same for a step of single tokens only (T == R tokens, request r at row q_start[r]),

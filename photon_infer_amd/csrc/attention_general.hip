@@ -1,4 +1,4 @@
-// Causal attention over the paged cache for any head size up to 256,
+// Causal attention over the paged cache for any head size up to 640 (a kernel for heads up to 256, one for wider ones),
 // any number of heads and groups, both storage types, prompts and single tokens alike.
 // One wave per (token, head); scores, softmax and the weighted sum are float32.
 //
@@ -29,16 +29,16 @@
 // ranges in range order with the same exact exponentials.
 #include "common.h"
 
-#define PI_MAX_HEAD_DIM 256
+#define PI_MAX_HEAD_DIM 640      // NACC = 4 serves heads up to 256, NACC = 10 up to 640
 
-template <typename T>
+template <typename T, int NACC>
 __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
     T* __restrict__ out, long out_stride, const T* __restrict__ q, long q_stride, const T* __restrict__ k_cache,
     const T* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ req_of_token, const int* __restrict__ positions, int nh, int nkv, int hd, int page_size,
     float scale, int window, long num_pages, float* __restrict__ part, int vd, const float* __restrict__ slopes,
     const float* __restrict__ sinks, const float* __restrict__ gate, float softcap, float out_mult, int chunk) {
-  __shared__ float qs[PI_MAX_HEAD_DIM];
+  __shared__ float qs[NACC * PI_WAVE];
   __shared__ float ps[PI_WAVE];
   __shared__ long voff[PI_WAVE];   // values are stored [page, kv_head, head_dim, slot]
   const long t = blockIdx.x;
@@ -52,7 +52,9 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
   if (chunk > 0 && (p / chunk) * chunk > lo) lo = (p / chunk) * chunk;
   const int* bt = block_table + (long)req_of_token[t] * table_width;
   float m = -INFINITY, l = 0.f;
-  float acc[PI_MAX_HEAD_DIM / PI_WAVE] = {0.f, 0.f, 0.f, 0.f};
+  float acc[NACC];
+#pragma unroll
+  for (int i = 0; i < NACC; ++i) acc[i] = 0.f;
   const float slope = slopes ? slopes[h] : 0.f;
   __syncthreads();
   // this wave's keys: all of lo..p, or the z-th of gridDim.z ranges of whole 64-key groups
@@ -100,7 +102,7 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
     ps[lane] = pe;
     voff[lane] = vo;
 #pragma unroll
-    for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) acc[i] *= corr;
+    for (int i = 0; i < NACC; ++i) acc[i] *= corr;
     __syncthreads();
     const int nk = (p - k0 + 1) < PI_WAVE ? (p - k0 + 1) : PI_WAVE;
     // keys in ascending order; four at a time where they lie side by side in a page (values are
@@ -113,7 +115,7 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
         if (four) {
           const float p0 = ps[kk], p1 = ps[kk + 1], p2 = ps[kk + 2], p3 = ps[kk + 3];
 #pragma unroll
-          for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) {
+          for (int i = 0; i < NACC; ++i) {
             const int d = lane + i * PI_WAVE;
             if (d < vd) {
               float vv[4];
@@ -127,7 +129,7 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
         } else {
           const float pk = ps[kk];
 #pragma unroll
-          for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) {
+          for (int i = 0; i < NACC; ++i) {
             const int d = lane + i * PI_WAVE;
             if (d < vd) acc[i] = fmaf(pk, to_float(vr[(long)d * page_size]), acc[i]);
           }
@@ -142,7 +144,7 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
     // [token, head, range, hd + 2]: the un-normalised sum, then the range's maximum and sum of weights
     float* mine = part + (((long)t * nh + h) * splits + blockIdx.z) * (vd + 2);
 #pragma unroll
-    for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) {
+    for (int i = 0; i < NACC; ++i) {
       const int d = lane + i * PI_WAVE;
       if (d < vd) mine[d] = acc[i];
     }
@@ -158,12 +160,12 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
     const float corr = expf(m - m_all);
     l = l * corr + expf(sk - m_all);
 #pragma unroll
-    for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) acc[i] *= corr;
+    for (int i = 0; i < NACC; ++i) acc[i] *= corr;
   }
   T* o = out + t * out_stride + (long)h * vd;
   const float inv = out_mult * (gate ? gate[t * nh + h] : 1.0f) / l;
 #pragma unroll
-  for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) {
+  for (int i = 0; i < NACC; ++i) {
     const int d = lane + i * PI_WAVE;
     if (d < vd) o[d] = from_float<T>(acc[i] * inv);
   }
@@ -171,7 +173,7 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
 
 // One wave per (token, head): o = sum_s e^(m_s - m) acc_s / sum_s e^(m_s - m) l_s, ranges in order;
 // an empty range (m_s = -inf, l_s = 0) counts nothing.
-template <typename T>
+template <typename T, int NACC>
 __global__ __launch_bounds__(PI_WAVE) void merge_key_ranges_kernel(T* __restrict__ out, long out_stride, const float* __restrict__ part,
                                                                    int nh, int hd, int splits, const float* __restrict__ sinks,
                                                                    const float* __restrict__ gate, float out_mult) {
@@ -181,13 +183,15 @@ __global__ __launch_bounds__(PI_WAVE) void merge_key_ranges_kernel(T* __restrict
   float m = sinks ? sinks[h] : -INFINITY;
   for (int s = 0; s < splits; ++s) m = fmaxf(m, base[s * (hd + 2) + hd]);
   float l = sinks ? expf(sinks[h] - m) : 0.f;
-  float acc[PI_MAX_HEAD_DIM / PI_WAVE] = {0.f, 0.f, 0.f, 0.f};
+  float acc[NACC];
+#pragma unroll
+  for (int i = 0; i < NACC; ++i) acc[i] = 0.f;
   for (int s = 0; s < splits; ++s) {
     const float ms = base[s * (hd + 2) + hd];
     const float w = ms == -INFINITY ? 0.f : expf(ms - m);
     l = fmaf(w, base[s * (hd + 2) + hd + 1], l);
 #pragma unroll
-    for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) {
+    for (int i = 0; i < NACC; ++i) {
       const int d = lane + i * PI_WAVE;
       if (d < hd) acc[i] = fmaf(w, base[s * (hd + 2) + d], acc[i]);
     }
@@ -195,7 +199,7 @@ __global__ __launch_bounds__(PI_WAVE) void merge_key_ranges_kernel(T* __restrict
   T* o = out + t * out_stride + (long)h * hd;
   const float inv = out_mult * (gate ? gate[t * nh + h] : 1.0f) / l;
 #pragma unroll
-  for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) {
+  for (int i = 0; i < NACC; ++i) {
     const int d = lane + i * PI_WAVE;
     if (d < hd) o[d] = from_float<T>(acc[i] * inv);
   }
@@ -231,12 +235,33 @@ extern "C" int pi_paged_attention_general(void* out, long out_stride, const void
   PI_REQUIRE(splits == 1 || (part && part_elems >= (long)T * nh * splits * (vd + 2)), "attention: workspace too small for %d key ranges", splits);
   if (T == 0) return 0;
   const dim3 grid(T, nh, splits), block(PI_WAVE);
+  const bool wide = hd > 256 || vd > 256;
+  if (wide) {
+#define PI_ATTN_WIDE 10
+    if (dtype == PI_F32)
+      hipLaunchKernelGGL((paged_attention_general_kernel<float, PI_ATTN_WIDE>), grid, block, 0, stream, (float*)out, out_stride, (const float*)q,
+                         q_stride, (const float*)k_cache, (const float*)v_cache, block_table, table_width, req_of_token,
+                         positions, nh, nkv, hd, page_size, scale, window, num_pages, (float*)part, vd, slopes, sinks, gate, softcap, out_mult, chunk);
+    else if (dtype == PI_BF16)
+      hipLaunchKernelGGL((paged_attention_general_kernel<bf16_t, PI_ATTN_WIDE>), grid, block, 0, stream, (bf16_t*)out, out_stride,
+                         (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width,
+                         req_of_token, positions, nh, nkv, hd, page_size, scale, window, num_pages, (float*)part, vd, slopes, sinks, gate, softcap, out_mult, chunk);
+    else
+      return pi_fail("attention: unsupported dtype %d", dtype);
+    if (pi_check_launch("paged_attention_general")) return -1;
+    if (splits == 1) return 0;
+    if (dtype == PI_F32)
+      hipLaunchKernelGGL((merge_key_ranges_kernel<float, PI_ATTN_WIDE>), dim3(T, nh), block, 0, stream, (float*)out, out_stride, (const float*)part, nh, vd, splits, sinks, gate, out_mult);
+    else
+      hipLaunchKernelGGL((merge_key_ranges_kernel<bf16_t, PI_ATTN_WIDE>), dim3(T, nh), block, 0, stream, (bf16_t*)out, out_stride, (const float*)part, nh, vd, splits, sinks, gate, out_mult);
+    return pi_check_launch("merge_key_ranges");
+  }
   if (dtype == PI_F32)
-    hipLaunchKernelGGL(paged_attention_general_kernel<float>, grid, block, 0, stream, (float*)out, out_stride, (const float*)q,
+    hipLaunchKernelGGL((paged_attention_general_kernel<float, 4>), grid, block, 0, stream, (float*)out, out_stride, (const float*)q,
                        q_stride, (const float*)k_cache, (const float*)v_cache, block_table, table_width, req_of_token,
                        positions, nh, nkv, hd, page_size, scale, window, num_pages, (float*)part, vd, slopes, sinks, gate, softcap, out_mult, chunk);
   else if (dtype == PI_BF16)
-    hipLaunchKernelGGL(paged_attention_general_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out, out_stride,
+    hipLaunchKernelGGL((paged_attention_general_kernel<bf16_t, 4>), grid, block, 0, stream, (bf16_t*)out, out_stride,
                        (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width,
                        req_of_token, positions, nh, nkv, hd, page_size, scale, window, num_pages, (float*)part, vd, slopes, sinks, gate, softcap, out_mult, chunk);
   else
@@ -244,8 +269,8 @@ extern "C" int pi_paged_attention_general(void* out, long out_stride, const void
   if (pi_check_launch("paged_attention_general")) return -1;
   if (splits == 1) return 0;
   if (dtype == PI_F32)
-    hipLaunchKernelGGL(merge_key_ranges_kernel<float>, dim3(T, nh), block, 0, stream, (float*)out, out_stride, (const float*)part, nh, vd, splits, sinks, gate, out_mult);
+    hipLaunchKernelGGL((merge_key_ranges_kernel<float, 4>), dim3(T, nh), block, 0, stream, (float*)out, out_stride, (const float*)part, nh, vd, splits, sinks, gate, out_mult);
   else
-    hipLaunchKernelGGL(merge_key_ranges_kernel<bf16_t>, dim3(T, nh), block, 0, stream, (bf16_t*)out, out_stride, (const float*)part, nh, vd, splits, sinks, gate, out_mult);
+    hipLaunchKernelGGL((merge_key_ranges_kernel<bf16_t, 4>), dim3(T, nh), block, 0, stream, (bf16_t*)out, out_stride, (const float*)part, nh, vd, splits, sinks, gate, out_mult);
   return pi_check_launch("merge_key_ranges");
 }

@@ -62,8 +62,19 @@ struct AttnOptions {
   const float* gate;
   float softcap = 0.f;
   float out_mult = 1.f;
+  int chunk = 0;          // C > 0: a token sees the keys of its own chunk of C positions only (a bound like the window's: no option of the arithmetic)
   bool any() const { return slopes || sinks || gate || softcap > 0.f || out_mult != 1.f; }
 };
+
+// The first key a token at position pos sees: 0, or pos - window + 1, or the start of pos's chunk (the later of them).
+__device__ inline int first_seen_key(int pos, int window, int chunk) {
+  int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  if (chunk > 0) {
+    const int c0 = pos - pos % chunk;
+    if (c0 > lo) lo = c0;
+  }
+  return lo;
+}
 
 // A raw score r (before the softmax scale) capped: (cap / scale) * tanh(r * scale / cap), with
 // tanh(x) = 1 - 2 / (1 + e^2x) from one v_exp_f32 and one v_rcp_f32; +-inf end at +-cap.

@@ -9,7 +9,7 @@
 // they share through LDS (stored in the very order the matrix-core operands want them, so
 // both the writes and the reads are 16 bytes per lane, lane after lane).  One barrier per 128
 // keys.  Heads of more than 128 features take 64 keys at a time (two of the waves fetch) and
-// 16 columns per wave: two rounds of 128 would not fit the LDS, nor the state the registers.  A token at absolute position p sees keys lo..p only (lo = 0, or p - window + 1),
+// 16 columns per wave: two rounds of 128 would not fit the LDS, nor the state the registers.  A token at absolute position p sees keys lo..p only (lo = 0, or p - window + 1, or the start of p's chunk),
 // whatever portion it arrived in; a wave skips the 32-key chunks none of its columns sees.
 //
 // The host sorts the tiles by the number of keys they walk and deals them out to the blocks
@@ -62,7 +62,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
     const int kv_len = kv_len_of[r];
     const int n_tok = min(TQ, q_len - q0);
     const int pos0 = kv_len - q_len + q0;          // position of the tile's first token
-    auto first_key = [&](int pos) { return (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0; };
+    auto first_key = [&](int pos) { return first_seen_key(pos, window, opt.chunk); };
     // keys the block walks: the tile's, or one of `cuts` equal shares of them in rounds of 128
     // (the host cuts the key range of tiles when a step has too few tiles for the chip; the
     // shares' results are merged by the combine kernel, as for decode attention)
@@ -218,7 +218,8 @@ extern "C" int pi_attention_prefill_mfma(void* out, long out_stride, const void*
                                          const int* tile_z0, void* part, const int* order, int rounds, int seats, int nh,
                                          int nkv, int hd, int page_size, float scale, int window, long num_pages,
                                          const float* slopes, const float* sinks, const float* gate, float softcap,
-                                         float out_mult, hipStream_t stream) {
+                                         float out_mult, int chunk, hipStream_t stream) {
+  PI_REQUIRE(chunk >= 0, "attention_prefill: chunk must be >= 0, got %d", chunk);
   PI_REQUIRE(rounds > 0 && seats > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_prefill: bad sizes rounds=%d seats=%d heads=%d kv_heads=%d", rounds, seats, nh, nkv);
   PI_REQUIRE(hd >= 16 && hd <= 256 && hd % 16 == 0, "attention_prefill: head_dim %d is not a multiple of 16 up to 256", hd);
   PI_REQUIRE(page_size >= 16 && page_size % 16 == 0, "attention_prefill: page size %d must be a multiple of 16", page_size);
@@ -229,7 +230,7 @@ extern "C" int pi_attention_prefill_mfma(void* out, long out_stride, const void*
   PI_REQUIRE(out_stride % 4 == 0 && q_stride % 8 == 0 && ((uintptr_t)q % 16 == 0) && ((uintptr_t)out % 8 == 0), "attention_prefill: q / out rows must be 16- / 8-byte aligned");
   const size_t lds = tiles_lds_bytes(hd);
   const dim3 grid(nkv, seats), block(256);
-  const AttnOptions opt{slopes, sinks, gate, softcap, out_mult};
+  const AttnOptions opt{slopes, sinks, gate, softcap, out_mult, chunk};
   const bool with_options = opt.any();
   PI_REQUIRE(!with_options || scale > 0.f, "attention_prefill: a distance bias or a cap needs a positive scale");
 #define GO(H, C, N)                    \

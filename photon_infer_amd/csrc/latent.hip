@@ -99,43 +99,58 @@ extern "C" int pi_latent_kv_write(void* cq_out, long cq_stride, int dtype, const
 // ---------------------------------------------------------------- a product per head
 // out[t, h * out_head + n] = sum_k a[t, h * a_head + k] * w[h, k, n]      (w: [heads, K, N], float32 sums in ascending k)
 // and, with `rot` > 0, the rot numbers that follow a head's K inputs are rotated by the token's angles (neighbouring pairs)
-// and placed behind the head's N results: [w_h^T a_h | rotate(tail)].  One block per (eight tokens, head): the tokens'
-// inputs sit in LDS, a thread owns output columns n, n + 256, ...; neighbouring threads read neighbouring weights.
-// A token's result does not depend on the tokens beside it.
+// and placed behind the head's N results: [w_h^T a_h | rotate(tail)].  One wave per (eight tokens, head, 64 output
+// columns): the tokens' inputs sit in LDS and are read four at a time, a lane owns one output column, neighbouring lanes
+// read neighbouring weights.  A token's result does not depend on the tokens beside it.
 #define HG_TOKENS 8
 template <typename T>
-__global__ __launch_bounds__(256) void head_gemm_kernel(T* __restrict__ out, long out_stride, int out_head, const T* __restrict__ a,
-                                                        long a_stride, int a_head, const T* __restrict__ w, int M, int K, int N,
-                                                        int rot, const float* __restrict__ table) {
-  extern __shared__ float as[];          // [HG_TOKENS][K + rot]
-  const int h = blockIdx.y;
+__global__ __launch_bounds__(PI_WAVE) void head_gemm_kernel(T* __restrict__ out, long out_stride, int out_head, const T* __restrict__ a,
+                                                            long a_stride, int a_head, const T* __restrict__ w, int M, int K, int N,
+                                                            int rot, const float* __restrict__ table) {
+  extern __shared__ __attribute__((aligned(16))) float as[];          // [HG_TOKENS][KP], KP = K + rot rounded up to four
+  const int h = blockIdx.y, lane = threadIdx.x;
   const long t0 = (long)blockIdx.x * HG_TOKENS;
   const int nt = (M - t0) < HG_TOKENS ? (int)(M - t0) : HG_TOKENS;
-  const int KR = K + rot;
-  for (int i = threadIdx.x; i < HG_TOKENS * KR; i += blockDim.x) {
-    const int tt = i / KR, k = i % KR;
-    as[i] = tt < nt ? to_float(a[(t0 + tt) * a_stride + (long)h * a_head + k]) : 0.f;
+  const int KR = K + rot, KP = (KR + 3) & ~3;
+  for (int i = lane; i < HG_TOKENS * KP; i += PI_WAVE) {
+    const int tt = i / KP, k = i % KP;
+    as[i] = (tt < nt && k < KR) ? to_float(a[(t0 + tt) * a_stride + (long)h * a_head + k]) : 0.f;
   }
   __syncthreads();
-  const T* wh = w + (long)h * K * N;
-  for (int n = threadIdx.x; n < N; n += blockDim.x) {
+  const int n = blockIdx.z * PI_WAVE + lane;
+  if (n < N) {
+    const T* wh = w + (long)h * K * N + n;
     float acc[HG_TOKENS];
 #pragma unroll
     for (int tt = 0; tt < HG_TOKENS; ++tt) acc[tt] = 0.f;
-    for (int k = 0; k < K; ++k) {
-      const float wv = to_float(wh[(long)k * N + n]);
+    int k = 0;
+    for (; k + 4 <= K; k += 4) {
+      const float w0 = to_float(wh[(long)k * N]), w1 = to_float(wh[(long)(k + 1) * N]);
+      const float w2 = to_float(wh[(long)(k + 2) * N]), w3 = to_float(wh[(long)(k + 3) * N]);
 #pragma unroll
-      for (int tt = 0; tt < HG_TOKENS; ++tt) acc[tt] = fmaf(as[tt * KR + k], wv, acc[tt]);
+      for (int tt = 0; tt < HG_TOKENS; ++tt) {
+        const float4 a4 = *reinterpret_cast<const float4*>(as + tt * KP + k);
+        acc[tt] = fmaf(a4.x, w0, acc[tt]);
+        acc[tt] = fmaf(a4.y, w1, acc[tt]);
+        acc[tt] = fmaf(a4.z, w2, acc[tt]);
+        acc[tt] = fmaf(a4.w, w3, acc[tt]);
+      }
+    }
+    for (; k < K; ++k) {
+      const float wv = to_float(wh[(long)k * N]);
+#pragma unroll
+      for (int tt = 0; tt < HG_TOKENS; ++tt) acc[tt] = fmaf(as[tt * KP + k], wv, acc[tt]);
     }
 #pragma unroll
     for (int tt = 0; tt < HG_TOKENS; ++tt)
       if (tt < nt) out[(t0 + tt) * out_stride + (long)h * out_head + n] = from_float<T>(acc[tt]);
   }
-  for (int i = threadIdx.x; i < nt * (rot / 2); i += blockDim.x) {
+  if (blockIdx.z != 0) return;
+  for (int i = lane; i < nt * (rot / 2); i += PI_WAVE) {
     const int tt = i / (rot / 2), j = i % (rot / 2);
     const float* cs = table + (t0 + tt) * rot;
     float lo, hi;
-    rope_pair(as[tt * KR + K + 2 * j], as[tt * KR + K + 2 * j + 1], cs[j], cs[rot / 2 + j], lo, hi);
+    rope_pair(as[tt * KP + K + 2 * j], as[tt * KP + K + 2 * j + 1], cs[j], cs[rot / 2 + j], lo, hi);
     T* o = out + (t0 + tt) * out_stride + (long)h * out_head + N;
     o[2 * j] = from_float<T>(lo);
     o[2 * j + 1] = from_float<T>(hi);
@@ -145,15 +160,15 @@ __global__ __launch_bounds__(256) void head_gemm_kernel(T* __restrict__ out, lon
 extern "C" int pi_head_gemm(void* out, long out_stride, int out_head, const void* a, long a_stride, int a_head, const void* w,
                             int dtype, int M, int heads, int K, int N, int rot, const float* table, hipStream_t stream) {
   PI_REQUIRE(M >= 0 && heads > 0 && K > 0 && N > 0 && rot >= 0 && rot % 2 == 0, "head product: bad sizes M=%d heads=%d K=%d N=%d rot=%d", M, heads, K, N, rot);
-  PI_REQUIRE(heads <= 65535, "head product: too many heads (%d)", heads);
+  PI_REQUIRE(heads <= 65535 && N <= 65535 * PI_WAVE, "head product: too many heads or columns (%d, %d)", heads, N);
   PI_REQUIRE(a_head >= K + rot && out_head >= N + rot, "head product: heads of %d / %d numbers hold no %d / %d", a_head, out_head, K + rot, N + rot);
   PI_REQUIRE(a_stride >= (long)(heads - 1) * a_head + K + rot && out_stride >= (long)(heads - 1) * out_head + N + rot,
              "head product: rows of %ld / %ld numbers hold no %d heads", a_stride, out_stride, heads);
   PI_REQUIRE(rot == 0 || table, "head product: a rotated tail needs the step's table");
-  const size_t lds = (size_t)HG_TOKENS * (K + rot) * sizeof(float);
+  const size_t lds = (size_t)HG_TOKENS * ((K + rot + 3) & ~3) * sizeof(float);
   PI_REQUIRE(lds <= 60000, "head product: %d inputs per head do not fit the staging memory", K + rot);
   if (M == 0) return 0;
-  const dim3 grid(ceil_div(M, HG_TOKENS), heads), block(256);
+  const dim3 grid(ceil_div(M, HG_TOKENS), heads, ceil_div(N, PI_WAVE)), block(PI_WAVE);
   if (dtype == PI_F32)
     hipLaunchKernelGGL(head_gemm_kernel<float>, grid, block, lds, stream, (float*)out, out_stride, out_head, (const float*)a, a_stride,
                        a_head, (const float*)w, M, K, N, rot, table);

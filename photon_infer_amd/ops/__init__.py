@@ -21,7 +21,8 @@ from . import _lib
 from .workspace import KernelWorkspace, KeyRanges, Partials, stream_layout, stream_layout_takes
 
 PI_F32, PI_BF16 = 0, 1
-MAX_HEAD_DIM = 256
+MAX_HEAD_DIM = 256              # the matrix-core attention kernels
+GENERAL_MAX_HEAD_DIM = 640      # the general attention kernel (key rows of a latent cache are wide)
 
 _FAST = True
 
@@ -93,8 +94,8 @@ def check_general_attention_sizes(num_heads: int, num_kv_heads: int, head_dim: i
     """Sizes the general attention kernel takes (the only one for heads with options)."""
     if num_heads <= 0 or num_kv_heads <= 0 or num_heads % num_kv_heads:
         raise KernelError(f"attention: {num_heads} heads is not a positive multiple of {num_kv_heads} kv heads")
-    if not (0 < head_dim <= MAX_HEAD_DIM and 0 < value_dim <= MAX_HEAD_DIM):
-        raise KernelError(f"attention: head sizes {head_dim} / {value_dim} must be at most {MAX_HEAD_DIM}")
+    if not (0 < head_dim <= GENERAL_MAX_HEAD_DIM and 0 < value_dim <= GENERAL_MAX_HEAD_DIM):
+        raise KernelError(f"attention: head sizes {head_dim} / {value_dim} must be at most {GENERAL_MAX_HEAD_DIM}")
 
 
 # ----------------------------------------------------------------------------- ops
@@ -521,12 +522,12 @@ def decode_length_bucket(max_kv_len: int) -> int:
 
 
 def attention_planner(dtype: torch.dtype, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int,
-                      window: int, device):
+                      window: int, device, chunk: int = 0):
     """What makes a step's work lists for an attention mixer of these sizes (a hashable object with
     ``plan(q_lens, kv_lens)``; equal ones share a plan), or None when its kernels need none."""
     if _FAST and dtype == torch.bfloat16 and _lib.build.MODULES["bf16"]:
         from . import fast
-        return fast.attention_planner(dtype, num_heads, num_kv_heads, head_dim, page_size, int(window), torch.device(device))
+        return fast.attention_planner(dtype, num_heads, num_kv_heads, head_dim, page_size, int(window), torch.device(device), int(chunk or 0))
     return None
 
 

@@ -347,13 +347,14 @@ class AttentionPlanner:
     singles_apart: bool       # requests that bring one token go to the key-split kernel instead
     units: int                # compute units of the device
     blocks_per_unit: int = 2  # blocks that a unit holds at a time (attention_blocks_per_unit)
+    chunk: int = 0            # C > 0: a token sees the keys of its own chunk of C positions only
 
     def plan(self, q_lens: Sequence[int], kv_lens: Sequence[int]):
         """None for a step of single tokens only (the key-split kernel needs no list); otherwise
         (int32 host arrays by name, a function from their device views to a ``TilePlan``)."""
         if self.singles_apart and all(n == 1 for n in q_lens):
             return None
-        tile_rows, window = self.tile_rows, self.window
+        tile_rows, window, chunk = self.tile_rows, self.window, self.chunk
         singles = tuple(r for r, n in enumerate(q_lens) if n == 1) if self.singles_apart else ()
         if len(singles) == len(q_lens):
             singles = ()
@@ -368,6 +369,8 @@ class AttentionPlanner:
                     first = kv - n + start                         # position of the tile's first token
                     last = first + min(tile_rows, n - start) - 1
                     lo = max(0, first - window + 1) if window > 0 else 0
+                    if chunk > 0:
+                        lo = max(lo, first - first % chunk)
                     walks.append(last // 128 - lo // 128 + 1)
                     first_row.append(row0 + start)
                     n_tok.append(min(tile_rows, n - start))
@@ -403,7 +406,7 @@ class AttentionPlanner:
 
 @functools.lru_cache(maxsize=None)
 def attention_planner(dtype, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, window: int,
-                      device) -> Optional[AttentionPlanner]:
+                      device, chunk: int = 0) -> Optional[AttentionPlanner]:
     """The planner for a mixer of these sizes, or None when the general kernel serves it."""
     if dtype != torch.bfloat16 or head_dim not in TILE_HEAD_DIMS or page_size % 16:
         return None
@@ -412,7 +415,7 @@ def attention_planner(dtype, num_heads: int, num_kv_heads: int, head_dim: int, p
         return None
     units = torch.cuda.get_device_properties(device).multi_processor_count
     return AttentionPlanner(tile_rows, int(window), num_kv_heads, num_heads // num_kv_heads <= 16, units,
-                            attention_blocks_per_unit(head_dim))
+                            attention_blocks_per_unit(head_dim), int(chunk))
 
 
 def upload_arrays(arrays: Dict[str, np.ndarray], device) -> Dict[str, torch.Tensor]:
@@ -520,15 +523,15 @@ def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_k
     """``slopes`` / ``sinks`` (float32 [heads]) and ``gate`` (float32 [tokens, heads]): a distance bias, a sink in
     the softmax and an output gate per head (None: none); ``softcap`` > 0: scaled scores s become
     softcap * tanh(s / softcap); ``out_scale``: a factor on every output."""
-    opt = tuple(None if t is None else t.data_ptr() for t in (slopes, sinks, gate)) + (float(softcap), float(out_scale))
-    if chunk:
-        return False
+    opt = tuple(None if t is None else t.data_ptr() for t in (slopes, sinks, gate)) + (float(softcap), float(out_scale), int(chunk))
     if head_dim not in DECODE_HEAD_DIMS or page_size % 16 or q.data_ptr() % 16 or q.stride(0) % 8 or out.stride(0) % 4:
         return False
     G = num_heads // num_kv_heads
     R = ctx.R
 
     def decode_kernel(n_req: int, req_ids: int, longest: int) -> None:
+        if chunk:                      # a token's keys end at its chunk's start, whatever the context
+            longest = min(longest, chunk)
         splits = _decode_splits_that_fit(ws, n_req, num_heads, num_kv_heads, head_dim, longest)
         part = _attn_part(ws, n_req * num_heads * splits * (head_dim + 4), q.device)
         _lib.call("bf16", "pi_attention_decode", out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0),
@@ -539,7 +542,7 @@ def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_k
     if ctx.all_decode and G <= 16:
         decode_kernel(R, 0, ctx.max_kv_len)
         return True
-    planner = attention_planner(q.dtype, num_heads, num_kv_heads, head_dim, page_size, window, q.device)
+    planner = attention_planner(q.dtype, num_heads, num_kv_heads, head_dim, page_size, window, q.device, int(chunk))
     if planner is None:
         return False
     # A step of prompt portions and single tokens: the single tokens, whose keys no other token

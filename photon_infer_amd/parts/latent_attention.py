@@ -70,9 +70,9 @@ class LatentAttention(Mixer):
 
     def value_rows(self, dtype) -> int:
         """Rows of a cached value page.  The latent alone is the value; where the matrix-core attention kernels can
-        serve the heads (bfloat16, a latent row that is a multiple of 16) the rotated part rides along, because those
+        serve the heads (bfloat16, a latent row that is a multiple of 16 up to their largest head) the rotated part rides along, because those
         kernels want values as wide as keys; what it adds to a head's result is never read."""
-        wide = dtype == torch.bfloat16 and self.latent_dim % 16 == 0 and ops.fast_kernels_enabled()
+        wide = dtype == torch.bfloat16 and self.latent_dim % 16 == 0 and self.latent_dim <= ops.MAX_HEAD_DIM and ops.fast_kernels_enabled()
         return self.latent_dim if wide else self.kv_rank
 
     def cache_spec(self):

@@ -100,6 +100,12 @@ class SinkWindowAttention(Mixer):
         return PagedCacheSpec((PagedTensor("k", (self.num_kv_heads, PAGE, self.head_dim)),
                                PagedTensor("v", (self.num_kv_heads, self.value_dim, PAGE))), self.cache_reach)
 
+    def step_planner(self, page_size: int):
+        if self.value_dim != self.head_dim or self.head_dim % 16:     # only the general kernel takes such heads; it needs no work lists
+            return None
+        return ops.attention_planner(self.dtype, self.num_heads, self.num_kv_heads, self.head_dim, page_size, self.window or 0,
+                                     self.device, self.chunk or 0)
+
     def load(self, tensors: Dict[str, torch.Tensor], dtype, device) -> None:
         super().load(tensors, dtype, device)
         mats = [tensors["q"]] + ([tensors["k"], tensors["v"]] if self.own_kv else []) + ([tensors["g"]] if self.output_gate else [])
