@@ -1,7 +1,7 @@
 #!/usr/bin/python3
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode1b|long1b|serve3b|mixed8b|dafidra|rorevik]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode1b|long1b|serve3b|mixed8b|dafidra|rorevik|dokanex]
                     [--batch 8,1,64] [--context 4096] [--dtype bf16|fp32]
 
 Every workload prints ONE JSON line.  The default, ``decode1b`` (Llama 3.2 1B layer sizes):  ``value`` is decoded tokens per second at batch 8 with the context
@@ -44,6 +44,11 @@ functions.  ``value`` is Dafidra's decoded tokens per second at the first size.
 ``--workload rorevik``: the Rorevik design (attention with capped scores beside a state-space mixer, a
 delta-rule memory in every third layer, clamped gated feed-forwards with biases) at layer sizes like
 Llama 3.2 1B's and 3B's, beside a Llama of the same width, depth and vocabulary, measured the same way.
+
+``--workload dokanex``: the Dokanex design (attention through a latent with a shared rotated key part; attention within
+chunks of 1,024 positions with unit heads, capped scores, a sink and a gate, every second such layer on the keys and
+values of the one before; a tied, capped head) at layer sizes like Llama 3.2 1B's and 3B's, beside a Llama of the same
+width, depth and vocabulary, measured the same way.
 
 Weights are random (N(0, 0.02), norms 1), token ids uniform random; no dataset is involved.
 """
@@ -585,6 +590,81 @@ def workload_rorevik(args) -> int:
     return 0
 
 
+def dokanex_config(width, heads, kv_heads, head_dim, ff, vocab, layers):
+    """A Dokanex of Llama-like layer sizes, layers in fours: two of attention through a latent (16 heads of 128 plain and
+    64 rotated query/key dimensions, a key/value latent of 192, so that a cached row holds 256 numbers, a query latent of
+    three eighths of the width, values as wide as fill the model's width; frequencies scaled by 8 over 1,024 positions), then
+    attention as the Llama's within chunks of 1,024 positions (unit heads, scores capped at 30, sink, gate), then the same
+    on the keys and values of the layer before it; dense gated feed-forwards of the Llama's width; logits capped at 30."""
+    lat = dict(heads=16, dim=128, rot_dim=64, vdim=width // 16, q_rank=width * 3 // 8, kv_rank=192, scale=192 ** -0.5,
+               rot={"base": 500000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}})
+    att = dict(heads=heads, kv_heads=kv_heads, dim=head_dim, vdim=head_dim, scale=head_dim ** -0.5, softcap=30.0, mask={"size": 1024})
+    mlp = {"kind": "dense", "ff": ff}
+    made = []
+    for i in range(layers):
+        if i % 4 < 2:
+            made.append({"type": "latent_attention", "mixer": lat, "mlp": mlp})
+        elif i % 4 == 2:
+            made.append({"type": "attention", "mixer": att, "mlp": mlp})
+        else:
+            made.append({"type": "attention", "mixer": dict(att, kv_from=i - 1), "mlp": mlp})
+    return {"architecture": "Dokanex", "vocab": vocab, "width": width, "embedding": {"scale": width ** 0.5}, "norm": {"eps": 1e-5},
+            "logit_softcap": 30.0, "layers": made}
+
+
+def workload_dokanex(args) -> int:
+    """Dokanex beside a Llama of equal width, depth and vocabulary (see the module text)."""
+    import gc
+
+    import torch
+
+    layers = args.layers or 4
+    context = args.context
+    positions = max(context, PREFILL_TOKENS) + 64
+    sizes = {"1b": MODEL, "3b": MODEL_3B}
+    results = {}
+
+    def config(b):
+        return dokanex_config(b["hidden_size"], b["num_attention_heads"], b["num_key_value_heads"], b["head_dim"],
+                              b["intermediate_size"], b["vocab_size"], layers)
+
+    if args.only:       # for profiles: the Dokanex of the first size alone, a prompt or decode steps
+        runner, _cfg = make_runner(config(sizes["1b"]), layers, args.dtype, args.batch, max(args.batch * (context + 64), PREFILL_TOKENS + 64),
+                                   max_model_len=positions)
+        if args.only == "prefill":
+            sec = time_prefill(runner, PREFILL_TOKENS, max(1, args.steps // 8))
+            print(json.dumps({"only": "prefill", "model": "dokanex_1b", "tokens": PREFILL_TOKENS, "ms": round(sec * 1e3, 3)}), flush=True)
+        else:
+            sec, _ = time_decode(runner, args.batch, args.steps, args.warmup, context, synthetic_cache=True)
+            print(json.dumps({"only": "decode", "model": "dokanex_1b", "batch": args.batch, "ms_per_step": round(sec * 1e3, 4),
+                              "cache": "random numbers, no prompt was run"}), flush=True)
+        return 0
+    for name, base in sizes.items():
+        for what, raw in (("dokanex", config(base)), ("llama", dict(base, tie_word_embeddings=False))):
+            runner, _cfg = make_runner(raw, layers, args.dtype, args.batch, max(args.batch * (context + 64), PREFILL_TOKENS + 64),
+                                       max_model_len=positions)
+            psec = time_prefill(runner, PREFILL_TOKENS, 3)
+            dsec, _ = time_decode(runner, args.batch, args.steps, args.warmup, context)
+            results[f"{what}_{name}"] = {"prefill_ms": round(psec * 1e3, 3), "prefill_tok_per_s": round(PREFILL_TOKENS / psec, 1),
+                                         "decode_ms_per_step": round(dsec * 1e3, 4), "decode_tok_per_s": round(args.batch / dsec, 1),
+                                         "graphs": len(runner._graphs)}
+            del runner
+            gc.collect()
+            torch.cuda.empty_cache()
+    first = results["dokanex_1b"]
+    line = {
+        "metric": f"decode tok/s at batch {args.batch}, context {context} (Dokanex at Llama 3.2 1B layer sizes, {layers} layers, random weights)",
+        "value": first["decode_tok_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": first["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
+        "config": {"model": "dokanex-at-llama-sizes", "layers": layers, "global_batch": args.batch, "seq_len": context,
+                   "prefill_tokens": PREFILL_TOKENS, "kv_block": BLOCK_SIZE, "parallelism": "single-gpu"},
+        "models": results,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -593,7 +673,7 @@ def main() -> int:
     ap.add_argument("--batch", default="8,1,64",
                     help="batch sizes of the decode steps: the first is the headline's, the others become points")
     ap.add_argument("--context", type=int, default=CONTEXT, help="context length that the decode steps end at")
-    ap.add_argument("--workload", choices=["decode1b", "long1b", "serve3b", "mixed8b", "dafidra", "rorevik"], default="decode1b")
+    ap.add_argument("--workload", choices=["decode1b", "long1b", "serve3b", "mixed8b", "dafidra", "rorevik", "dokanex"], default="decode1b")
     ap.add_argument("--layers", type=int, default=None,
                     help="fewer layers than the model has, if memory or time needs it (both numbers are reported)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
@@ -629,6 +709,8 @@ def main() -> int:
         return workload_dafidra(args)
     if args.workload == "rorevik":
         return workload_rorevik(args)
+    if args.workload == "dokanex":
+        return workload_dokanex(args)
     args.layers = args.layers or MODEL["num_hidden_layers"]
     elem = 2 if args.dtype == "bf16" else 4
     big = args.batch if (args.no_points or args.only) else max(batches)

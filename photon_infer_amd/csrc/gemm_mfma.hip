@@ -172,7 +172,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
                                                         const bf16_t* __restrict__ W, long ldw, int M, int N, int K,
                                                         int tiles_n, int k_per_split, const int* __restrict__ group_of_tile,
                                                         const int* __restrict__ tile_row0, const int* __restrict__ tile_rows,
-                                                        long group_stride, GluArgs glu) {
+                                                        long group_stride, long group_a_step, long group_c_step, GluArgs glu) {
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
   constexpr int ROW = BK;                   // rows of 128 bytes, no padding (see the large-tile kernel)
   constexpr int TILE = BM * ROW;
@@ -201,7 +201,9 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
   // Grouped: the rows are sorted by group (a routed feed-forward's experts) and cut into tiles of
   // up to 128 rows of one group; tile t multiplies rows tile_row0[t] .. + tile_rows[t] - 1 with the
   // matrix of group group_of_tile[t] (W + group * group_stride).  The list lives on the device
-  // and is as long as the worst case; unused entries (-1) end their blocks at once.
+  // and is as long as the worst case; unused entries (-1) end their blocks at once.  A group may also sit
+  // at columns of its own in A and C (group * group_a_step, group * group_c_step elements into a row): a product
+  // per head, whose heads lie side by side in the rows.
   if (group_of_tile) {
     const int t = blockIdx.x / tiles_n;
     const int grp = group_of_tile[t];
@@ -210,9 +212,9 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
     tile_m = 0;
     tile_n = blockIdx.x % tiles_n;
     M = tile_rows[t];
-    A += r0 * lda;
+    A += r0 * lda + grp * group_a_step;
     W += (long)grp * group_stride;
-    Cv = reinterpret_cast<char*>(Cv) + r0 * ldc * (EPI == EPI_BF16 || EPI_GATED(EPI) ? 2 : 4);
+    Cv = reinterpret_cast<char*>(Cv) + (r0 * ldc + grp * group_c_step) * (EPI == EPI_BF16 || EPI_GATED(EPI) ? 2 : 4);
   }
   const long m0 = (long)tile_m * BM, n0 = (long)tile_n * BN;
 
@@ -536,7 +538,7 @@ static int launch(void* C, long ldc, const void* A, long lda, const void* W, lon
   const int tiles_m = ceil_div(M, BM), tiles_n = ceil_div(N, BN);
   hipLaunchKernelGGL((gemm_mfma_kernel<EPI>), dim3((unsigned)tiles_m * tiles_n, splits), dim3(256), kLdsBytes, stream, C, ldc,
                      (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, tiles_n, kps, (const int*)nullptr, (const int*)nullptr,
-                     (const int*)nullptr, 0L, glu);
+                     (const int*)nullptr, 0L, 0L, 0L, glu);
   return pi_check_launch("gemm_mfma");
 }
 
@@ -549,7 +551,7 @@ extern "C" int pi_gemm_mfma_group_tile_rows() { return BM; }
 template <int EPI>
 static int launch_grouped(void* C, long ldc, const void* A, long lda, const void* W, long ldw, long group_stride,
                           const int* group_of_tile, const int* tile_row0, const int* tile_rows, int tiles, int N, int K,
-                          hipStream_t stream) {
+                          long group_a_step, long group_c_step, hipStream_t stream) {
   static bool configured = false;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_mfma_kernel<EPI>),
@@ -560,14 +562,17 @@ static int launch_grouped(void* C, long ldc, const void* A, long lda, const void
   const int tiles_n = ceil_div(N, BN);
   hipLaunchKernelGGL((gemm_mfma_kernel<EPI>), dim3((unsigned)tiles * tiles_n, 1), dim3(256), kLdsBytes, stream, C, ldc,
                      (const bf16_t*)A, lda, (const bf16_t*)W, ldw, BM, N, K, tiles_n, K, group_of_tile, tile_row0, tile_rows,
-                     group_stride, GluArgs{nullptr, 0.f, 0.f});
+                     group_stride, group_a_step, group_c_step, GluArgs{nullptr, 0.f, 0.f});
   return pi_check_launch("gemm_mfma_grouped");
 }
 
 extern "C" int pi_gemm_mfma_grouped(void* C, int epilogue, long ldc, const void* A, long lda, const void* W, long ldw,
                                     long group_stride, const int* group_of_tile, const int* tile_row0, const int* tile_rows,
-                                    int tiles, int N, int K, hipStream_t stream) {
+                                    int tiles, int N, int K, long group_a_step, long group_c_step, hipStream_t stream) {
   PI_REQUIRE(tiles >= 0 && N > 0 && K > 0, "gemm_mfma_grouped: bad sizes tiles=%d N=%d K=%d", tiles, N, K);
+  PI_REQUIRE(group_a_step >= 0 && group_c_step >= 0 && group_a_step % 8 == 0 && group_c_step % 8 == 0,
+             "gemm_mfma_grouped: a group's columns in the rows (%ld, %ld) must start at multiples of 8", group_a_step, group_c_step);
+  PI_REQUIRE(group_c_step == 0 || epilogue == EPI_BF16 || epilogue == EPI_F32, "gemm_mfma_grouped: groups side by side in the result's rows store plainly");
   PI_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && group_stride % 8 == 0, "gemm_mfma_grouped: K (%d) and strides must be multiples of 8", K);
   PI_REQUIRE(256 * lda < (1L << 29) && 256 * ldw < (1L << 29), "gemm_mfma_grouped: row strides (%ld, %ld) are too long", lda, ldw);
   PI_REQUIRE(ldc > 0 && ldc < (1L << 23), "gemm_mfma_grouped: the result's row stride (%ld) is too long", ldc);
@@ -577,9 +582,9 @@ extern "C" int pi_gemm_mfma_grouped(void* C, int epilogue, long ldc, const void*
   PI_REQUIRE(group_of_tile && tile_row0 && tile_rows, "gemm_mfma_grouped: the tile list is missing");
   if (tiles == 0) return 0;
   switch (epilogue) {
-    case EPI_BF16: return launch_grouped<EPI_BF16>(C, ldc, A, lda, W, ldw, group_stride, group_of_tile, tile_row0, tile_rows, tiles, N, K, stream);
-    case EPI_F32: return launch_grouped<EPI_F32>(C, ldc, A, lda, W, ldw, group_stride, group_of_tile, tile_row0, tile_rows, tiles, N, K, stream);
-    case EPI_SWIGLU: return launch_grouped<EPI_SWIGLU>(C, ldc, A, lda, W, ldw, group_stride, group_of_tile, tile_row0, tile_rows, tiles, N, K, stream);
+    case EPI_BF16: return launch_grouped<EPI_BF16>(C, ldc, A, lda, W, ldw, group_stride, group_of_tile, tile_row0, tile_rows, tiles, N, K, group_a_step, group_c_step, stream);
+    case EPI_F32: return launch_grouped<EPI_F32>(C, ldc, A, lda, W, ldw, group_stride, group_of_tile, tile_row0, tile_rows, tiles, N, K, group_a_step, group_c_step, stream);
+    case EPI_SWIGLU: return launch_grouped<EPI_SWIGLU>(C, ldc, A, lda, W, ldw, group_stride, group_of_tile, tile_row0, tile_rows, tiles, N, K, group_a_step, group_c_step, stream);
   }
   return pi_fail("gemm_mfma_grouped: unknown epilogue %d", epilogue);
 }

@@ -97,56 +97,81 @@ extern "C" int pi_latent_kv_write(void* cq_out, long cq_stride, int dtype, const
 }
 
 // ---------------------------------------------------------------- a product per head
-// out[t, h * out_head + n] = sum_k a[t, h * a_head + k] * w[h, k, n]      (w: [heads, K, N], float32 sums in ascending k)
+// out[t, h * out_head + n] = sum_k a[t, h * a_head + k] * w[h, k, n]      (w: [heads, K, N])
 // and, with `rot` > 0, the rot numbers that follow a head's K inputs are rotated by the token's angles (neighbouring pairs)
-// and placed behind the head's N results: [w_h^T a_h | rotate(tail)].  One wave per (eight tokens, head, 64 output
-// columns): the tokens' inputs sit in LDS and are read four at a time, a lane owns one output column, neighbouring lanes
-// read neighbouring weights.  A token's result does not depend on the tokens beside it.
+// and placed behind the head's N results: [w_h^T a_h | rotate(tail)].  One block per (eight tokens, head, 64 output
+// columns): the tokens' inputs sit in LDS and are read four at a time; a lane owns one output column, neighbouring lanes
+// read neighbouring weights, eight loads in flight; the block's four waves each take a quarter of k (in whole eights) and
+// their float32 sums - each in ascending k - are added in wave order.  A token's result does not depend on the tokens
+// beside it.  `skip_product`: only the rotated tails are made (the product comes from another kernel).
 #define HG_TOKENS 8
+#define HG_WAVES 4
 template <typename T>
-__global__ __launch_bounds__(PI_WAVE) void head_gemm_kernel(T* __restrict__ out, long out_stride, int out_head, const T* __restrict__ a,
-                                                            long a_stride, int a_head, const T* __restrict__ w, int M, int K, int N,
-                                                            int rot, const float* __restrict__ table) {
+__global__ __launch_bounds__(HG_WAVES * PI_WAVE) void head_gemm_kernel(T* __restrict__ out, long out_stride, int out_head,
+                                                                       const T* __restrict__ a, long a_stride, int a_head,
+                                                                       const T* __restrict__ w, int M, int K, int N, int rot,
+                                                                       const float* __restrict__ table, int skip_product) {
   extern __shared__ __attribute__((aligned(16))) float as[];          // [HG_TOKENS][KP], KP = K + rot rounded up to four
-  const int h = blockIdx.y, lane = threadIdx.x;
+  __shared__ float sums[HG_WAVES][HG_TOKENS][PI_WAVE];
+  const int h = blockIdx.y, lane = threadIdx.x % PI_WAVE, wave = threadIdx.x / PI_WAVE;
   const long t0 = (long)blockIdx.x * HG_TOKENS;
   const int nt = (M - t0) < HG_TOKENS ? (int)(M - t0) : HG_TOKENS;
   const int KR = K + rot, KP = (KR + 3) & ~3;
-  for (int i = lane; i < HG_TOKENS * KP; i += PI_WAVE) {
+  const int k_from = skip_product ? K : 0;
+  for (int i = threadIdx.x; i < HG_TOKENS * KP; i += blockDim.x) {
     const int tt = i / KP, k = i % KP;
-    as[i] = (tt < nt && k < KR) ? to_float(a[(t0 + tt) * a_stride + (long)h * a_head + k]) : 0.f;
+    as[i] = (tt < nt && k >= k_from && k < KR) ? to_float(a[(t0 + tt) * a_stride + (long)h * a_head + k]) : 0.f;
   }
   __syncthreads();
-  const int n = blockIdx.z * PI_WAVE + lane;
-  if (n < N) {
-    const T* wh = w + (long)h * K * N + n;
+  if (!skip_product) {
+    const int n = blockIdx.z * PI_WAVE + lane;
+    const int per = ((K + HG_WAVES - 1) / HG_WAVES + 7) & ~7;          // a wave's share of k, in whole eights
+    const int k0 = wave * per, k1 = min(K, k0 + per);
     float acc[HG_TOKENS];
 #pragma unroll
     for (int tt = 0; tt < HG_TOKENS; ++tt) acc[tt] = 0.f;
-    int k = 0;
-    for (; k + 4 <= K; k += 4) {
-      const float w0 = to_float(wh[(long)k * N]), w1 = to_float(wh[(long)(k + 1) * N]);
-      const float w2 = to_float(wh[(long)(k + 2) * N]), w3 = to_float(wh[(long)(k + 3) * N]);
+    if (n < N) {
+      const T* wh = w + (long)h * K * N + n;
+      int k = k0;
+      for (; k + 8 <= k1; k += 8) {
+        float wv[8];
 #pragma unroll
-      for (int tt = 0; tt < HG_TOKENS; ++tt) {
-        const float4 a4 = *reinterpret_cast<const float4*>(as + tt * KP + k);
-        acc[tt] = fmaf(a4.x, w0, acc[tt]);
-        acc[tt] = fmaf(a4.y, w1, acc[tt]);
-        acc[tt] = fmaf(a4.z, w2, acc[tt]);
-        acc[tt] = fmaf(a4.w, w3, acc[tt]);
+        for (int u = 0; u < 8; ++u) wv[u] = to_float(wh[(long)(k + u) * N]);
+#pragma unroll
+        for (int tt = 0; tt < HG_TOKENS; ++tt) {
+          const float4 a0 = *reinterpret_cast<const float4*>(as + tt * KP + k);
+          const float4 a1 = *reinterpret_cast<const float4*>(as + tt * KP + k + 4);
+          acc[tt] = fmaf(a0.x, wv[0], acc[tt]);
+          acc[tt] = fmaf(a0.y, wv[1], acc[tt]);
+          acc[tt] = fmaf(a0.z, wv[2], acc[tt]);
+          acc[tt] = fmaf(a0.w, wv[3], acc[tt]);
+          acc[tt] = fmaf(a1.x, wv[4], acc[tt]);
+          acc[tt] = fmaf(a1.y, wv[5], acc[tt]);
+          acc[tt] = fmaf(a1.z, wv[6], acc[tt]);
+          acc[tt] = fmaf(a1.w, wv[7], acc[tt]);
+        }
+      }
+      for (; k < k1; ++k) {
+        const float wv = to_float(wh[(long)k * N]);
+#pragma unroll
+        for (int tt = 0; tt < HG_TOKENS; ++tt) acc[tt] = fmaf(as[tt * KP + k], wv, acc[tt]);
       }
     }
-    for (; k < K; ++k) {
-      const float wv = to_float(wh[(long)k * N]);
 #pragma unroll
-      for (int tt = 0; tt < HG_TOKENS; ++tt) acc[tt] = fmaf(as[tt * KP + k], wv, acc[tt]);
+    for (int tt = 0; tt < HG_TOKENS; ++tt) sums[wave][tt][lane] = acc[tt];
+    __syncthreads();
+    // wave tt (and tt + 4) finishes token tt: the four shares in wave order
+    for (int tt = wave; tt < nt; tt += HG_WAVES) {
+      if (n < N) {
+        float v = sums[0][tt][lane];
+#pragma unroll
+        for (int u = 1; u < HG_WAVES; ++u) v += sums[u][tt][lane];
+        out[(t0 + tt) * out_stride + (long)h * out_head + n] = from_float<T>(v);
+      }
     }
-#pragma unroll
-    for (int tt = 0; tt < HG_TOKENS; ++tt)
-      if (tt < nt) out[(t0 + tt) * out_stride + (long)h * out_head + n] = from_float<T>(acc[tt]);
   }
   if (blockIdx.z != 0) return;
-  for (int i = lane; i < nt * (rot / 2); i += PI_WAVE) {
+  for (int i = threadIdx.x; i < nt * (rot / 2); i += blockDim.x) {
     const int tt = i / (rot / 2), j = i % (rot / 2);
     const float* cs = table + (t0 + tt) * rot;
     float lo, hi;
@@ -158,23 +183,25 @@ __global__ __launch_bounds__(PI_WAVE) void head_gemm_kernel(T* __restrict__ out,
 }
 
 extern "C" int pi_head_gemm(void* out, long out_stride, int out_head, const void* a, long a_stride, int a_head, const void* w,
-                            int dtype, int M, int heads, int K, int N, int rot, const float* table, hipStream_t stream) {
+                            int dtype, int M, int heads, int K, int N, int rot, const float* table, int skip_product,
+                            hipStream_t stream) {
   PI_REQUIRE(M >= 0 && heads > 0 && K > 0 && N > 0 && rot >= 0 && rot % 2 == 0, "head product: bad sizes M=%d heads=%d K=%d N=%d rot=%d", M, heads, K, N, rot);
   PI_REQUIRE(heads <= 65535 && N <= 65535 * PI_WAVE, "head product: too many heads or columns (%d, %d)", heads, N);
   PI_REQUIRE(a_head >= K + rot && out_head >= N + rot, "head product: heads of %d / %d numbers hold no %d / %d", a_head, out_head, K + rot, N + rot);
   PI_REQUIRE(a_stride >= (long)(heads - 1) * a_head + K + rot && out_stride >= (long)(heads - 1) * out_head + N + rot,
              "head product: rows of %ld / %ld numbers hold no %d heads", a_stride, out_stride, heads);
   PI_REQUIRE(rot == 0 || table, "head product: a rotated tail needs the step's table");
+  PI_REQUIRE(skip_product || w, "head product: the weights are missing");
   const size_t lds = (size_t)HG_TOKENS * ((K + rot + 3) & ~3) * sizeof(float);
-  PI_REQUIRE(lds <= 60000, "head product: %d inputs per head do not fit the staging memory", K + rot);
-  if (M == 0) return 0;
-  const dim3 grid(ceil_div(M, HG_TOKENS), heads, ceil_div(N, PI_WAVE)), block(PI_WAVE);
+  PI_REQUIRE(lds <= 48000, "head product: %d inputs per head do not fit the staging memory", K + rot);
+  if (M == 0 || (skip_product && rot == 0)) return 0;
+  const dim3 grid(ceil_div(M, HG_TOKENS), heads, skip_product ? 1 : ceil_div(N, PI_WAVE)), block(HG_WAVES * PI_WAVE);
   if (dtype == PI_F32)
     hipLaunchKernelGGL(head_gemm_kernel<float>, grid, block, lds, stream, (float*)out, out_stride, out_head, (const float*)a, a_stride,
-                       a_head, (const float*)w, M, K, N, rot, table);
+                       a_head, (const float*)w, M, K, N, rot, table, skip_product);
   else if (dtype == PI_BF16)
     hipLaunchKernelGGL(head_gemm_kernel<bf16_t>, grid, block, lds, stream, (bf16_t*)out, out_stride, out_head, (const bf16_t*)a, a_stride,
-                       a_head, (const bf16_t*)w, M, K, N, rot, table);
+                       a_head, (const bf16_t*)w, M, K, N, rot, table, skip_product);
   else
     return pi_fail("head product: unsupported dtype %d", dtype);
   return pi_check_launch("head_gemm");

@@ -666,13 +666,15 @@ def latent_kv_write(cq_out: Optional[torch.Tensor], proj, w_q: Optional[torch.Te
 
 
 def head_gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, heads: int, a_head: Optional[int] = None,
-              out_head: Optional[int] = None, rot: int = 0, table: Optional[torch.Tensor] = None) -> None:
+              out_head: Optional[int] = None, rot: int = 0, table: Optional[torch.Tensor] = None,
+              w_rows: Optional[torch.Tensor] = None) -> None:
     """A product per head: ``out[t, h * out_head + n] = sum_k a[t, h * a_head + k] * w[h, k, n]`` with ``w``
     [heads, K, N] (a head's matrix stored with its inputs as rows), float32 sums.  ``a_head`` / ``out_head``: the
     distance between two heads in a row of ``a`` / ``out`` (default K + rot / N + rot).  ``rot`` > 0: the ``rot`` numbers
     behind a head's K inputs are turned by the token's angles (``table``: the step's [T, rot] cosines and sines,
-    neighbouring pairs) and placed behind the head's N results."""
-    _gpu(out, a, w, table)
+    neighbouring pairs) and placed behind the head's N results.  ``w_rows``: the same matrices stored [heads, N, K]
+    (a head's outputs as rows), which the matrix-core kernel reads for steps of many tokens (bfloat16)."""
+    _gpu(out, a, w, table, w_rows)
     if w.dim() != 3 or w.shape[0] != heads or not w.is_contiguous():
         raise KernelError(f"head product: weights must be contiguous [{heads}, K, N], got {tuple(w.shape)}")
     K, N = int(w.shape[1]), int(w.shape[2])
@@ -685,12 +687,19 @@ def head_gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, heads: int, a
         raise KernelError(f"head product: rows of {a.shape[1]} / {out.shape[1]} numbers do not hold {heads} heads of {a_head} / {out_head}")
     if rot and (table is None or table.shape != (M, rot) or table.dtype != torch.float32 or not table.is_contiguous()):
         raise KernelError(f"head product: cos / sin table must be contiguous float32 [{M}, {rot}]")
-    if _FAST and a.dtype == torch.bfloat16 and rot == 0:
+    if M == 0:
+        return
+    skip = 0
+    if _FAST and a.dtype == torch.bfloat16 and w_rows is not None:
+        if w_rows.shape != (heads, N, K) or w_rows.dtype != a.dtype or not w_rows.is_contiguous():
+            raise KernelError(f"head product: the row-major weights must be contiguous [{heads}, {N}, {K}] {a.dtype}")
         from . import fast
-        if fast.head_gemm(out, a, w, heads, K, N, a_head, out_head):
-            return
+        if fast.head_gemm(out, a, w_rows, heads, K, N, a_head, out_head, _rows(a, "head product a"), _rows(out, "head product out")):
+            if rot == 0:
+                return
+            skip = 1          # the rotated tails are still to make
     _lib.call("core", "pi_head_gemm", out.data_ptr(), _rows(out, "head product out"), out_head, a.data_ptr(), _rows(a, "head product a"),
-              a_head, w.data_ptr(), _dt(a), M, heads, K, N, int(rot), _ptr(table), _stream())
+              a_head, w.data_ptr(), _dt(a), M, heads, K, N, int(rot), _ptr(table), skip, _stream())
 
 
 # ----------------------------------------------------------------------------- matrix memory
@@ -827,7 +836,7 @@ def _grouped_fast(out, a, w, rows: ExpertRows, epilogue: int) -> bool:
         return False
     _lib.call("bf16", "pi_gemm_mfma_grouped", out.data_ptr(), epilogue, _rows(out, "out"), a.data_ptr(), _rows(a, "a"), w.data_ptr(),
               K, w.shape[1] * K, rows.tile_expert.data_ptr(), rows.tile_row0.data_ptr(), rows.tile_rows.data_ptr(),
-              rows.tile_expert.numel(), w.shape[1], K, _stream())
+              rows.tile_expert.numel(), w.shape[1], K, 0, 0, _stream())
     return True
 
 

@@ -32,7 +32,7 @@ _SIGNATURES = {
         "pi_cast_stream": [P, I, P, L, P],
         "pi_qk_norm_kv_write": [P, L, P, I, P, L, P, P, P, P, F, F, I, I, I, I, I, I, I, P, P, P, I, I, L, P, I, L, I, I, P],
         "pi_latent_kv_write": [P, L, I, P, L, P, P, P, P, P, F, I, I, I, I, I, P, P, P, I, I, L, P, I, L, P],
-        "pi_head_gemm": [P, L, I, P, L, I, P, I, I, I, I, I, I, P, P],
+        "pi_head_gemm": [P, L, I, P, L, I, P, I, I, I, I, I, I, P, I, P],
         "pi_matrix_memory_scan": [P, L, P, L, I, I, I, I, I, P, P, F, F, P, P, I, P, L, I, I, I, I, I, I, P, L, P],
         "pi_head_norm_gate": [P, I, P, L, P, L, P, F, I, I, I, F, P],
         "pi_route": [P, P, P, L, I, I, I, I, I, I, P],
@@ -49,7 +49,7 @@ _SIGNATURES = {
         "pi_gemm_mfma": [P, I, L, P, L, P, L, I, I, I, I, P],
         "pi_gemm_mfma_pieces": [I, I],
         "pi_gemm_mfma_clamped_glu": [P, L, P, L, P, L, I, I, I, P, F, F, P],
-        "pi_gemm_mfma_grouped": [P, I, L, P, L, P, L, L, P, P, P, I, I, I, P],
+        "pi_gemm_mfma_grouped": [P, I, L, P, L, P, L, L, P, P, P, I, I, I, L, L, P],
         "pi_gemm_skinny": [P, I, L, P, L, P, L, I, I, I, I, P, L, P, I, P],
         "pi_splitk_reduce": [P, I, L, P, I, I, I, P],
         "pi_attention_tile_rows": [I, I, I],

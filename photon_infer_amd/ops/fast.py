@@ -303,9 +303,33 @@ def gemm_clamped_glu(out, a, w, bias, limit, alpha, M, N, K, lda, ldw) -> bool:
     return True
 
 
-def head_gemm(out, a, w, heads: int, K: int, N: int, a_head: int, out_head: int) -> bool:
-    """A product per head on the matrix-core kernels; False: not for these sizes."""
-    return False
+HEAD_TILES_FROM_TOKENS = 129   # a product per head takes the grouped tile kernel from this many tokens on
+
+
+@functools.lru_cache(maxsize=64)
+def _head_tiles(M: int, heads: int, device) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """The grouped tile kernel's list for a product per head: head h's rows are all M rows, cut into tiles of 128."""
+    rows = _lib.load("bf16").pi_gemm_mfma_group_tile_rows()
+    starts = np.arange(0, M, rows, dtype=np.int32)
+    group = np.repeat(np.arange(heads, dtype=np.int32), len(starts))
+    row0 = np.tile(starts, heads)
+    count = np.minimum(rows, M - row0).astype(np.int32)
+    return tuple(torch.from_numpy(x).to(device) for x in (group, row0, count))
+
+
+def head_gemm(out, a, w_rows, heads: int, K: int, N: int, a_head: int, out_head: int, lda: int, ldc: int) -> bool:
+    """A product per head (``w_rows`` [heads, N, K]) as one launch of the grouped tile kernel, every head a group that
+    sits at columns of its own in the rows of ``a`` and ``out``; False: not for these sizes (few tokens, or heads that
+    do not start at multiples of 8 columns)."""
+    M = a.shape[0]
+    if M < HEAD_TILES_FROM_TOKENS or K % 8 or lda % 8 or a_head % 8 or out_head % 8 or a.data_ptr() % 16 or w_rows.data_ptr() % 16:
+        return False
+    if 256 * lda >= (1 << 29) or ldc >= (1 << 23) or out.data_ptr() % 4:
+        return False
+    group, row0, count = _head_tiles(M, heads, a.device)
+    _lib.call("bf16", "pi_gemm_mfma_grouped", out.data_ptr(), EPI_BF16, ldc, a.data_ptr(), lda, w_rows.data_ptr(), K, N * K,
+              group.data_ptr(), row0.data_ptr(), count.data_ptr(), group.numel(), N, K, a_head, out_head, _stream())
+    return True
 
 
 # ----------------------------------------------------------------------------- attention

@@ -101,6 +101,10 @@ class LatentAttention(Mixer):
         # coordinates come out) and W_uv_n transposed ([kv_rank, value_dim]: the attended latent goes in)
         self.w_uk = tensors[n[5]].to(dtype).reshape(H, d, r).contiguous()
         self.w_uv = tensors[n[6]].to(dtype).reshape(H, dv, r).transpose(1, 2).contiguous()
+        # and with outputs as rows, which the matrix-core kernel reads for steps of many tokens
+        fast = dtype == torch.bfloat16 and ops.fast_kernels_enabled()
+        self.w_uk_rows = self.w_uk.transpose(1, 2).contiguous() if fast else None
+        self.w_uv_rows = tensors[n[6]].to(dtype).reshape(H, dv, r).contiguous() if fast else None
         self.w_o = tensors[n[7]]
         if self.position is not None:
             self.position.load({}, dtype, device)
@@ -121,7 +125,7 @@ class LatentAttention(Mixer):
         ops.gemm(q, cq, self.w_uq, ws=ws)
         # queries in the latent's coordinates, the rotated part behind them
         q_lat = torch.empty((T, H * self.latent_dim), dtype=self.dtype, device=h.device)
-        ops.head_gemm(q_lat, q, self.w_uk, H, rot=self.rot_dim, table=rot_table)
+        ops.head_gemm(q_lat, q, self.w_uk, H, rot=self.rot_dim, table=rot_table, w_rows=self.w_uk_rows)
         v_rows = cache.v.shape[2]
         att = torch.empty((T, H * v_rows), dtype=self.dtype, device=h.device)
         if v_rows == self.latent_dim:
@@ -130,7 +134,7 @@ class LatentAttention(Mixer):
             ops.paged_attention(att, q_lat, cache.k, cache.v, table, ctx, H, 1, self.latent_dim, cache.page_size, self.scale, 0, ws,
                                 value_dim=v_rows)
         out = torch.empty((T, self.o_size), dtype=self.dtype, device=h.device)
-        ops.head_gemm(out, att, self.w_uv, H, a_head=v_rows)
+        ops.head_gemm(out, att, self.w_uv, H, a_head=v_rows, w_rows=self.w_uv_rows)
         ops.gemm(x, out, self.w_o, accumulate=self.accumulate,
                  may_defer=self.accumulate and getattr(ctx, "may_defer", False), ws=ws)
 

@@ -216,12 +216,15 @@ def test_scaled_rotation_table_and_the_ramp_ends():
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("sizes", [(1, 3, 24, 30, 0), (9, 4, 16, 24, 8), (77, 2, 128, 200, 16), (8, 5, 7, 65, 2), (130, 1, 64, 64, 0)])
+@pytest.mark.parametrize("sizes", [(1, 3, 24, 30, 0), (9, 4, 16, 24, 8), (77, 2, 128, 200, 16), (8, 5, 7, 65, 2), (130, 1, 64, 64, 0),
+                                   (300, 3, 64, 96, 16), (257, 4, 40, 72, 0)])
 def test_a_product_per_head_with_a_rotated_tail(dtype, sizes):
+    """Few tokens take the general kernel; in bfloat16, from 129 tokens on, heads that start at multiples of 8 columns take
+    the matrix-core kernel (one launch, every head a group at columns of its own), the rotated tails a launch of their own."""
     from photon_infer_amd import ops
     M, H, K, N, rot = sizes
     tdt = TORCH[dtype]
-    a, w = randn(M, H * (K + rot) + 3, seed=1).to(tdt), randn(H, K, N, seed=2).to(tdt)
+    a, w = randn(M, H * (K + rot) + (8 if M > 128 else 3), seed=1).to(tdt), randn(H, K, N, seed=2).to(tdt)
     freqs = [0.37 ** i for i in range(rot // 2)]
     pos = torch.arange(M) * 3
     want = torch.zeros((M, H, N + rot), dtype=F64)
@@ -232,7 +235,8 @@ def test_a_product_per_head_with_a_rotated_tail(dtype, sizes):
         want[..., N:] = P.rotate_pairs(ah[..., K:], pos, freqs, 1.3)
         table = ops.rope_table(pos.to(torch.int32).to(DEV), torch.tensor(freqs, dtype=torch.float32, device=DEV), 1.3)
     out = torch.full((M, H * (N + rot) + 5), 7.0, dtype=tdt, device=DEV)
-    ops.head_gemm(out, a.to(DEV), w.to(DEV).contiguous(), H, rot=rot, table=table)
+    rows = w.transpose(1, 2).contiguous().to(DEV) if dtype == "bfloat16" else None
+    ops.head_gemm(out, a.to(DEV), w.to(DEV).contiguous(), H, rot=rot, table=table, w_rows=rows)
     close(out[:, :H * (N + rot)], want.reshape(M, -1), f"{sizes}", 2e-5 if dtype == "float32" else 2e-2)
     assert bool((out[:, H * (N + rot):] == 7.0).all())
 
