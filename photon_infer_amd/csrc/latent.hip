@@ -101,11 +101,12 @@ extern "C" int pi_latent_kv_write(void* cq_out, long cq_stride, int dtype, const
 // and, with `rot` > 0, the rot numbers that follow a head's K inputs are rotated by the token's angles (neighbouring pairs)
 // and placed behind the head's N results: [w_h^T a_h | rotate(tail)].  One block per (eight tokens, head, 64 output
 // columns): the tokens' inputs sit in LDS and are read four at a time; a lane owns one output column, neighbouring lanes
-// read neighbouring weights, eight loads in flight; the block's four waves each take a quarter of k (in whole eights) and
+// read neighbouring weights, sixteen loads in flight; the block's eight waves each take an eighth of k (in whole eights) and
 // their float32 sums - each in ascending k - are added in wave order.  A token's result does not depend on the tokens
 // beside it.  `skip_product`: only the rotated tails are made (the product comes from another kernel).
 #define HG_TOKENS 8
-#define HG_WAVES 4
+#define HG_WAVES 8
+#define HG_LOADS 16        // weights a lane asks for before it waits: a wave's whole share of k at the usual sizes
 template <typename T>
 __global__ __launch_bounds__(HG_WAVES * PI_WAVE) void head_gemm_kernel(T* __restrict__ out, long out_stride, int out_head,
                                                                        const T* __restrict__ a, long a_stride, int a_head,
@@ -133,6 +134,22 @@ __global__ __launch_bounds__(HG_WAVES * PI_WAVE) void head_gemm_kernel(T* __rest
     if (n < N) {
       const T* wh = w + (long)h * K * N + n;
       int k = k0;
+      for (; k + HG_LOADS <= k1; k += HG_LOADS) {
+        float wv[HG_LOADS];
+#pragma unroll
+        for (int u = 0; u < HG_LOADS; ++u) wv[u] = to_float(wh[(long)(k + u) * N]);
+#pragma unroll
+        for (int tt = 0; tt < HG_TOKENS; ++tt) {
+#pragma unroll
+          for (int u = 0; u < HG_LOADS; u += 4) {
+            const float4 a4 = *reinterpret_cast<const float4*>(as + tt * KP + k + u);
+            acc[tt] = fmaf(a4.x, wv[u], acc[tt]);
+            acc[tt] = fmaf(a4.y, wv[u + 1], acc[tt]);
+            acc[tt] = fmaf(a4.z, wv[u + 2], acc[tt]);
+            acc[tt] = fmaf(a4.w, wv[u + 3], acc[tt]);
+          }
+        }
+      }
       for (; k + 8 <= k1; k += 8) {
         float wv[8];
 #pragma unroll
@@ -160,7 +177,7 @@ __global__ __launch_bounds__(HG_WAVES * PI_WAVE) void head_gemm_kernel(T* __rest
 #pragma unroll
     for (int tt = 0; tt < HG_TOKENS; ++tt) sums[wave][tt][lane] = acc[tt];
     __syncthreads();
-    // wave tt (and tt + 4) finishes token tt: the four shares in wave order
+    // wave tt finishes token tt: the waves' shares in wave order
     for (int tt = wave; tt < nt; tt += HG_WAVES) {
       if (n < N) {
         float v = sums[0][tt][lane];
