@@ -155,7 +155,8 @@ def test_a_lone_key_beside_the_sink_in_closed_form():
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("sizes", [(2, 16, 8, 24, 20, 24), (4, 32, 16, 32, 64, 48), (3, 20, 6, 28, 10, 30), (1, 24, 16, 40, 32, 272), (5, 8, 2, 8, 8, 8)])
+@pytest.mark.parametrize("sizes", [(2, 16, 8, 24, 20, 24), (4, 32, 16, 32, 64, 48), (3, 20, 6, 28, 10, 30), (1, 24, 16, 40, 32, 272), (5, 8, 2, 8, 8, 8),
+                                   (20, 8, 8, 8, 16, 24), (16, 16, 16, 16, 32, 112)])
 def test_latent_attention_mixer_whole_in_portions_and_token_by_token(dtype, sizes):
     """The mixer as a part on pages dealt out of order: a prompt whole, then in portions, then its end token by token; the
     rotation's frequencies are scaled over an original length that the prompt passes.  One latent far back is loud."""
