@@ -475,7 +475,7 @@ __device__ inline void attn_walk(AttnState<HD, CB>& st, int c0, int c1, int firs
     meanwhile();
     return;
   }
-  KVChunk<HD> a, b;
+  KVChunk<HD> a;
   KVLaneOffsets<HD> off;
   off.set(page_size, lane);
   const int num_pages = (int)(num_pages_l < 0x7fffffffL ? num_pages_l : 0x7fffffffL);
@@ -486,6 +486,21 @@ __device__ inline void attn_walk(AttnState<HD, CB>& st, int c0, int c1, int firs
   // them: the loads of one buffer are then always the youngest in flight when the other is
   // consumed, which lets the compiler wait by count.  Up to two chunks beyond the range are
   // loaded and never used.
+  if constexpr (HD > 192) {
+    // Heads this wide: one chunk's keys and values are 128 registers, two chunks in flight beside the accumulators
+    // do not fit the register file (the kernel spilled to memory).  One buffer: a chunk is asked for when the one
+    // before it has been used; page ids still run a chunk ahead.
+    ChunkPages pn = cur.next();
+    attn_load<HD>(a, pn, k_cache, v_cache, off, nkv, g, page_size, num_pages);
+    meanwhile();
+    for (int c = c0; c < c1; ++c) {
+      pn = cur.next();
+      attn_compute<HD, CB, KVChunk<HD>, BIAS>(st, a, c * 32, scale_log2, c < first_unmasked || c > last_unmasked, lane);
+      if (c + 1 < c1) attn_load<HD>(a, pn, k_cache, v_cache, off, nkv, g, page_size, num_pages);
+    }
+    return;
+  }
+  KVChunk<HD> b;
   ChunkPages pa = cur.next(), pb = cur.next();
   attn_load<HD>(a, pa, k_cache, v_cache, off, nkv, g, page_size, num_pages);
   meanwhile();
