@@ -291,6 +291,31 @@ extern "C" int pi_swiglu(void* out, const void* gu, int dtype, int T, int I, int
   return pi_check_launch("swiglu");
 }
 
+// ------------------------------------------------------------------ squared relu
+// out = max(in, 0)^2, from the float32 results of a product into the activation type: the square is
+// taken before the one rounding.
+template <typename TO>
+__global__ void relu_squared_kernel(TO* __restrict__ out, const float* __restrict__ in, long n) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float v = fmaxf(in[i], 0.f);
+  out[i] = from_float<TO>(v * v);
+}
+
+extern "C" int pi_relu_squared(void* out, int out_dtype, const float* in, long n, hipStream_t stream) {
+  PI_REQUIRE(n >= 0 && out && in, "squared relu: bad arguments");
+  if (n == 0) return 0;
+  const long blocks = (n + 255) / 256;
+  PI_REQUIRE(blocks < 2147483647L, "squared relu: too many elements (%ld)", n);
+  if (out_dtype == PI_F32)
+    hipLaunchKernelGGL(relu_squared_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, stream, (float*)out, in, n);
+  else if (out_dtype == PI_BF16)
+    hipLaunchKernelGGL(relu_squared_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, (bf16_t*)out, in, n);
+  else
+    return pi_fail("squared relu: unsupported dtype %d", out_dtype);
+  return pi_check_launch("relu_squared");
+}
+
 // ------------------------------------------------------------------ clamped gated unit with biases
 // g = min(gate + bg, limit), u = clamp(up + bu, -limit, limit), out = g * sigmoid(alpha * g) * (u + 1).
 // The gate and up products lie in halves of a row ([gate | up]) in TI; biases and arithmetic are
@@ -374,9 +399,10 @@ extern "C" int pi_rope_table(float* table, const int* positions, const float* in
 // [splits, T, ncols] with q at column q_col, k at k_col, v at v_col; the rotated q then goes to
 // the q buffer, and nothing ever holds the unrotated values in reduced precision.
 template <typename T>
-__device__ inline float rope_source(const T* __restrict__ src, const float* __restrict__ part, int splits, long part_stride, int i) {
-  if (!part) return to_float(src[i]);
-  return split_sum(part, splits, part_stride, i);
+__device__ inline float rope_source(const T* __restrict__ src, const float* __restrict__ part, int splits, long part_stride, int i,
+                                    const float* __restrict__ bias = nullptr) {
+  const float v = part ? split_sum(part, splits, part_stride, i) : to_float(src[i]);
+  return bias ? v + bias[i] : v;      // the projection's bias, by column
 }
 
 // One wave per (token, head), four heads to a block; a lane owns whole pairs, so nothing is
@@ -387,7 +413,8 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
     const int* __restrict__ positions, const int* __restrict__ req_of_token, const float* __restrict__ table,
     int rotary_dim, int interleaved, int nh, int nkv_write, int nkv, int hd, T* __restrict__ k_cache,
     T* __restrict__ v_cache, const int* __restrict__ block_table, int table_width, int page_size, long num_pages,
-    const float* __restrict__ part, int splits, long part_stride, int ncols, int q_col, int k_col, int v_col, int vd) {
+    const float* __restrict__ part, int splits, long part_stride, int ncols, int q_col, int k_col, int v_col, int vd,
+    const float* __restrict__ bias) {
   const long t = blockIdx.x;
   const int h = blockIdx.y * 4 + threadIdx.x / PI_WAVE;
   const int lane = threadIdx.x % PI_WAVE;
@@ -426,23 +453,24 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
     }
   }
   const float* pp = part ? part + t * ncols + col : nullptr;
+  const float* bp = bias ? bias + col : nullptr;
   if (rotate) {
     const int half = rotary_dim / 2;
     for (int j = lane; j < half; j += PI_WAVE) {
       const int i0 = interleaved ? 2 * j : j;
       const int i1 = interleaved ? 2 * j + 1 : j + half;
-      const float a = rope_source(src, pp, splits, part_stride, i0);
-      const float b = rope_source(src, pp, splits, part_stride, i1);
+      const float a = rope_source(src, pp, splits, part_stride, i0, bp);
+      const float b = rope_source(src, pp, splits, part_stride, i1, bp);
       const float c = table[t * rotary_dim + j], s = table[t * rotary_dim + half + j];
       float lo, hi;
       rope_pair(a, b, c, s, lo, hi);
       dst[i0 * dst_stride] = from_float<T>(lo);
       dst[i1 * dst_stride] = from_float<T>(hi);
     }
-    if (part || dst != src)
-      for (int i = rotary_dim + lane; i < hd; i += PI_WAVE) dst[i * dst_stride] = from_float<T>(rope_source(src, pp, splits, part_stride, i));
-  } else if (part || dst != src) {
-    for (int i = lane; i < width; i += PI_WAVE) dst[i * dst_stride] = from_float<T>(rope_source(src, pp, splits, part_stride, i));
+    if (part || bp || dst != src)
+      for (int i = rotary_dim + lane; i < hd; i += PI_WAVE) dst[i * dst_stride] = from_float<T>(rope_source(src, pp, splits, part_stride, i, bp));
+  } else if (part || bp || dst != src) {
+    for (int i = lane; i < width; i += PI_WAVE) dst[i * dst_stride] = from_float<T>(rope_source(src, pp, splits, part_stride, i, bp));
   }
 }
 
@@ -579,7 +607,8 @@ extern "C" int pi_rope_kv_write(void* q, long q_stride, const void* k, long k_st
                                 int rotary_dim, int interleaved, int T, int nh, int nkv, int hd, int write_kv,
                                 void* k_cache, void* v_cache, const int* block_table, int table_width,
                                 int page_size, long num_pages, const float* part, int splits, int ncols, int q_col,
-                                int k_col, int v_col, int vd, hipStream_t stream) {
+                                int k_col, int v_col, int vd, const float* bias, hipStream_t stream) {
+  // bias: float32, one per column of the projection [q heads | k heads | v heads], found at q_col / k_col / v_col
   if (vd <= 0) vd = hd;
   PI_REQUIRE(vd <= 256, "rope_kv_write: value width %d must be at most 256", vd);
   PI_REQUIRE(T >= 0 && nh >= 0 && nkv >= 0 && hd > 0 && hd <= 256, "rope_kv_write: bad sizes T=%d heads=%d kv_heads=%d head_dim=%d", T, nh, nkv, hd);
@@ -598,7 +627,7 @@ extern "C" int pi_rope_kv_write(void* q, long q_stride, const void* k, long k_st
                               : (!write_kv || (k_stride % 8 == 0 && ((uintptr_t)k % 16 == 0)));
   const bool aligned = hd % 16 == 0 && q_stride % 8 == 0 && ((uintptr_t)q % 16 == 0) && (!table || (uintptr_t)table % 16 == 0) &&
                        source_ok && (!write_kv || (((uintptr_t)k_cache % 16 == 0) && ((uintptr_t)v_cache % 8 == 0) && page_size % 4 == 0));
-  if (dtype == PI_BF16 && usual && aligned && T >= 16 && vd == hd) {
+  if (dtype == PI_BF16 && usual && aligned && T >= 16 && vd == hd && !bias) {
     const int nkv_w = write_kv ? nkv : 0;
     const long rot_items = (long)T * (nh + nkv_w) * (hd / 16);
     const long v_items = write_kv ? (long)((T + 3) / 4) * nkv * hd : 0;
@@ -618,12 +647,12 @@ extern "C" int pi_rope_kv_write(void* q, long q_stride, const void* k, long k_st
     hipLaunchKernelGGL(rope_kv_write_kernel<float>, grid, block, 0, stream, (float*)q, q_stride, (const float*)k, k_stride,
                        (const float*)v, v_stride, positions, req_of_token, table, rotary_dim, interleaved, nh, nkv_write,
                        nkv, hd, (float*)k_cache, (float*)v_cache, block_table, table_width, page_size, num_pages, part,
-                       splits, part_stride, ncols, q_col, k_col, v_col, vd);
+                       splits, part_stride, ncols, q_col, k_col, v_col, vd, bias);
   else if (dtype == PI_BF16)
     hipLaunchKernelGGL(rope_kv_write_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)q, q_stride, (const bf16_t*)k, k_stride,
                        (const bf16_t*)v, v_stride, positions, req_of_token, table, rotary_dim, interleaved, nh, nkv_write,
                        nkv, hd, (bf16_t*)k_cache, (bf16_t*)v_cache, block_table, table_width, page_size, num_pages, part,
-                       splits, part_stride, ncols, q_col, k_col, v_col, vd);
+                       splits, part_stride, ncols, q_col, k_col, v_col, vd, bias);
   else
     return pi_fail("rope_kv_write: unsupported dtype %d", dtype);
   return pi_check_launch("rope_kv_write");

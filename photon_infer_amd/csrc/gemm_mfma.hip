@@ -30,7 +30,10 @@ PI_DEFINE_MODULE(bf16)
 #define BK 64
 #define TILE_ELEMS (BM * BK)                // a tile's slab in LDS: rows of 128 bytes
 
-enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACCUM = 2, EPI_SWIGLU = 3, EPI_CLAMPED_GLU = 4 };
+enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACCUM = 2, EPI_SWIGLU = 3, EPI_CLAMPED_GLU = 4, EPI_RELU2 = 5 };
+
+// results that leave as bfloat16, one per input column: as they are, or through max(c, 0)^2
+#define EPI_HALF(E) ((E) == EPI_BF16 || (E) == EPI_RELU2)
 
 // the gated epilogues store one output column per pair of input columns, in bfloat16
 #define EPI_GATED(E) ((E) == EPI_SWIGLU || (E) == EPI_CLAMPED_GLU)
@@ -113,14 +116,21 @@ __device__ inline void store_rows32(float* patch, const f32x16_t& acc0, const f3
           if (j * 32 + 16 + q * 8 + e < cols_left) dst[e] = from_float<bf16_t>(o[e]);
       }
     }
-  } else if (EPI == EPI_BF16) {
+  } else if (EPI_HALF(EPI)) {
     bf16_t* out = reinterpret_cast<bf16_t*>(C);
 #pragma unroll
     for (int pass = 0; pass < 4; ++pass) {
       const int id = pass * 64 + lane, r = id / 8, c = (id % 8) * 8;
       if (row0 + r >= rows_left || c >= cols_left) continue;
       const float* src = patch + r * PATCH_LD + c;
-      const f32x4_t a = *reinterpret_cast<const f32x4_t*>(src), b = *reinterpret_cast<const f32x4_t*>(src + 4);
+      f32x4_t a = *reinterpret_cast<const f32x4_t*>(src), b = *reinterpret_cast<const f32x4_t*>(src + 4);
+      if (EPI == EPI_RELU2) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          a[e] = fmaxf(a[e], 0.f); a[e] *= a[e];
+          b[e] = fmaxf(b[e], 0.f); b[e] *= b[e];
+        }
+      }
       bf16_t* dst = out + (row0 + r) * ld + c;
       if (wide && c + 8 <= cols_left) {
         *reinterpret_cast<u32x4_t*>(dst) = u32x4_t{pack2(a[0], a[1]), pack2(a[2], a[3]), pack2(b[0], b[1]), pack2(b[2], b[3])};
@@ -214,7 +224,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
     M = tile_rows[t];
     A += r0 * lda + grp * group_a_step;
     W += (long)grp * group_stride;
-    Cv = reinterpret_cast<char*>(Cv) + (r0 * ldc + grp * group_c_step) * (EPI == EPI_BF16 || EPI_GATED(EPI) ? 2 : 4);
+    Cv = reinterpret_cast<char*>(Cv) + (r0 * ldc + grp * group_c_step) * (EPI_HALF(EPI) || EPI_GATED(EPI) ? 2 : 4);
   }
   const long m0 = (long)tile_m * BM, n0 = (long)tile_n * BN;
 
@@ -331,7 +341,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
     const long mw = m0 + wm * 64, nw = n0 + wn * 64;
     const int rows_left = (int)min((long)64, M - mw), cols_left = (int)min((long)64, N - nw);   // may be <= 0
     float* patch = reinterpret_cast<float*>(lds) + wave * PATCH_FLOATS;
-    const int esize = EPI == EPI_BF16 || EPI_GATED(EPI) ? 2 : 4;
+    const int esize = EPI_HALF(EPI) || EPI_GATED(EPI) ? 2 : 4;
     char* corner = reinterpret_cast<char*>(Cv) + (mw * ldc + (EPI_GATED(EPI) ? nw / 2 : nw)) * esize;
     const bool wide = (ldc * esize) % 16 == 0 && reinterpret_cast<uintptr_t>(corner) % 16 == 0;
 #pragma unroll
@@ -486,7 +496,7 @@ __global__ __launch_bounds__(512) void gemm_mfma_big_kernel(void* __restrict__ C
     const long mw = m0 + wm * 128, nw = n0 + wn * 64;
     const int rows_left = (int)min((long)128, M - mw), cols_left = (int)min((long)64, N - nw);   // may be <= 0
     float* patch = reinterpret_cast<float*>(lds) + wave * PATCH_FLOATS;
-    const int esize = EPI == EPI_BF16 || EPI_GATED(EPI) ? 2 : 4;
+    const int esize = EPI_HALF(EPI) || EPI_GATED(EPI) ? 2 : 4;
     char* corner = reinterpret_cast<char*>(Cv) + (mw * ldc + (EPI_GATED(EPI) ? nw / 2 : nw)) * esize;
     const bool wide = (ldc * esize) % 16 == 0 && reinterpret_cast<uintptr_t>(corner) % 16 == 0;
 #pragma unroll
@@ -584,6 +594,7 @@ extern "C" int pi_gemm_mfma_grouped(void* C, int epilogue, long ldc, const void*
   switch (epilogue) {
     case EPI_BF16: return launch_grouped<EPI_BF16>(C, ldc, A, lda, W, ldw, group_stride, group_of_tile, tile_row0, tile_rows, tiles, N, K, group_a_step, group_c_step, stream);
     case EPI_F32: return launch_grouped<EPI_F32>(C, ldc, A, lda, W, ldw, group_stride, group_of_tile, tile_row0, tile_rows, tiles, N, K, group_a_step, group_c_step, stream);
+    case EPI_RELU2: return launch_grouped<EPI_RELU2>(C, ldc, A, lda, W, ldw, group_stride, group_of_tile, tile_row0, tile_rows, tiles, N, K, group_a_step, group_c_step, stream);
     case EPI_SWIGLU: return launch_grouped<EPI_SWIGLU>(C, ldc, A, lda, W, ldw, group_stride, group_of_tile, tile_row0, tile_rows, tiles, N, K, group_a_step, group_c_step, stream);
   }
   return pi_fail("gemm_mfma_grouped: unknown epilogue %d", epilogue);
@@ -595,7 +606,8 @@ extern "C" int pi_gemm_mfma_pieces(int K, int splits) {
   return addressing::cut_k(K, splits, BK).splits;
 }
 
-// epilogue: 0 store bf16, 1 store f32, 2 add into f32, 3 SwiGLU (W rows interleaved by 16; C is [M, N / 2] bf16)
+// epilogue: 0 store bf16, 1 store f32, 2 add into f32, 3 SwiGLU (W rows interleaved by 16; C is [M, N / 2] bf16),
+// 5 store max(c, 0)^2 as bf16
 extern "C" int pi_gemm_mfma(void* C, int epilogue, long ldc, const void* A, long lda, const void* W, long ldw, int M,
                             int N, int K, int splits, hipStream_t stream) {
   PI_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_mfma: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -613,6 +625,7 @@ extern "C" int pi_gemm_mfma(void* C, int epilogue, long ldc, const void* A, long
     case EPI_BF16: return launch<EPI_BF16>(C, ldc, A, lda, W, ldw, M, N, K, splits, stream);
     case EPI_F32: return launch<EPI_F32>(C, ldc, A, lda, W, ldw, M, N, K, splits, stream);
     case EPI_ACCUM: return launch<EPI_ACCUM>(C, ldc, A, lda, W, ldw, M, N, K, splits, stream);
+    case EPI_RELU2: return launch<EPI_RELU2>(C, ldc, A, lda, W, ldw, M, N, K, splits, stream);
     case EPI_SWIGLU: return launch<EPI_SWIGLU>(C, ldc, A, lda, W, ldw, M, N, K, splits, stream);
   }
   return pi_fail("gemm_mfma: unknown epilogue %d", epilogue);

@@ -370,11 +370,13 @@ extern "C" int pi_matrix_memory_scan(float* out, long out_stride, const float* p
   return pi_check_launch("matrix_memory_scan");
 }
 
-// y[t, h*dv + c] = o / sqrt(mean_c(o^2) + eps) * w[h*dv + c] * sigmoid(g[t, h*dv + c]); one wave per (token, head)
+// y[t, h*dv + c] = o / sqrt(mean_c(o^2) + eps) * w[h*dv + c] * act(g[t, h*dv + c]); one wave per (token, head);
+// act: the sigmoid, or (silu_gate) z * sigmoid(z)
 template <typename T>
 __global__ __launch_bounds__(PI_WAVE) void head_norm_gate_kernel(T* __restrict__ y, const float* __restrict__ o, long o_stride,
                                                                  const float* __restrict__ g, long g_stride,
-                                                                 const float* __restrict__ w, float eps, int heads, int dv, float mult) {
+                                                                 const float* __restrict__ w, float eps, int heads, int dv, float mult,
+                                                                 int silu_gate) {
   const long t = blockIdx.x;
   const int h = blockIdx.y, lane = threadIdx.x;
   const float* orow = o + t * o_stride + (long)h * dv;
@@ -382,20 +384,22 @@ __global__ __launch_bounds__(PI_WAVE) void head_norm_gate_kernel(T* __restrict__
   for (int c = lane; c < dv; c += PI_WAVE) ss = fmaf(orow[c], orow[c], ss);
   const float r = mult / sqrtf(wave_sum(ss) / dv + eps);
   for (int c = lane; c < dv; c += PI_WAVE) {
-    const float gate = 1.0f / (1.0f + expf(-g[t * g_stride + h * dv + c]));
+    const float z = g[t * g_stride + h * dv + c];
+    const float sg = 1.0f / (1.0f + expf(-z));
+    const float gate = silu_gate ? z * sg : sg;
     y[(t * heads + h) * dv + c] = from_float<T>(orow[c] * r * w[h * dv + c] * gate);
   }
 }
 
 extern "C" int pi_head_norm_gate(void* y, int dtype, const float* o, long o_stride, const float* g, long g_stride,
-                                 const float* w, float eps, int T, int heads, int dv, float mult, hipStream_t stream) {
+                                 const float* w, float eps, int T, int heads, int dv, float mult, int silu_gate, hipStream_t stream) {
   PI_REQUIRE(T >= 0 && heads > 0 && heads <= 65535 && dv > 0, "head norm: bad sizes");
   if (T == 0) return 0;
   const dim3 grid(T, heads), block(PI_WAVE);
   if (dtype == PI_F32)
-    hipLaunchKernelGGL(head_norm_gate_kernel<float>, grid, block, 0, stream, (float*)y, o, o_stride, g, g_stride, w, eps, heads, dv, mult);
+    hipLaunchKernelGGL(head_norm_gate_kernel<float>, grid, block, 0, stream, (float*)y, o, o_stride, g, g_stride, w, eps, heads, dv, mult, silu_gate);
   else if (dtype == PI_BF16)
-    hipLaunchKernelGGL(head_norm_gate_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)y, o, o_stride, g, g_stride, w, eps, heads, dv, mult);
+    hipLaunchKernelGGL(head_norm_gate_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)y, o, o_stride, g, g_stride, w, eps, heads, dv, mult, silu_gate);
   else
     return pi_fail("head norm: unsupported dtype %d", dtype);
   return pi_check_launch("head_norm_gate");

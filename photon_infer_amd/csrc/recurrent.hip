@@ -1,6 +1,6 @@
 // Mixers whose memory is a state of fixed size per request: the short causal convolution in
 // front of them, the state-space recurrence (Mamba-2 form), the gated delta rule with one decay
-// per head and key channel, and the norms behind them.  Everything that enters a recurrence is
+// per head and key channel or per head, gated linear attention, and the norms behind them.  Everything that enters a recurrence is
 // float32 in both compute modes: inputs after the convolution, step sizes, decays, gates, the
 // state.  A request's state row lies at state[slots[r]]; a step runs the tokens
 // q_start[r] .. q_start[r+1]-1 of request r from that row and leaves the row ready for the next
@@ -347,23 +347,36 @@ extern "C" int pi_gated_group_norm(void* out, int out_dtype, long out_stride, co
   return pi_check_launch("gated_group_norm");
 }
 
-// ------------------------------------------------------------------ gated delta rule, a decay per key channel
-// Per head h with key head g = h / (H / G), state S [d, dv] (float32, zero at the start):
-//   q^ = q / sqrt(sum q^2 + unit_eps) * q_scale;  k^ = k / sqrt(sum k^2 + unit_eps);
-//   decay[c] = exp(-exp(A_log[h]) * softplus(a[h, c] + dt_bias[h, c]));  beta = sigmoid(b[h]);
-//   S <- diag(decay) S;  u = beta * (v - S^T k^);  S <- S + k^ u^T;  o = S^T q^
-// q, k, v are columns of the convolution's output (q at 0, k at G * d, v at 2 * G * d).
+// ------------------------------------------------------------------ walks over a state with decayed key rows
+// Per head h with key head g = h / (H / G), state S [d, dv] (float32, zero at the start).  Three kinds:
+//   SCAN_CHANNEL_DELTA  the gated delta rule with a decay per head and key channel:
+//     q^ = q / sqrt(sum q^2 + unit_eps) * q_scale;  k^ = k / sqrt(sum k^2 + unit_eps);
+//     decay[c] = exp(-exp(A_log[h]) * softplus(a[h, c] + dt_bias[h, c]));  beta = sigmoid(b[h]);
+//     S <- diag(decay) S;  u = beta * (v - S^T k^);  S <- S + k^ u^T;  o = S^T q^
+//   SCAN_HEAD_DELTA     the same with one decay per head: a is [T, H], dt_bias [H],
+//     decay = exp(-exp(A_log[h]) * softplus(a[h] + dt_bias[h]));  S <- decay S
+//   SCAN_DECAYED_OUTER  gated linear attention, no delta term and no unit vectors:
+//     q' = q * q_scale;  decay[c] = sigmoid(a[h, c] + dt_bias[h, c])^(1 / tau);
+//     S <- diag(decay) S + k v^T;  o = S^T q'
+// q, k, v are columns of one float32 row per token (q at 0, k at G * d, v at 2 * G * d).
 //
-// First, once per token and head and in place: unit vectors over q and k, decays over a, beta over b.
-// One wave per (token, key head) and per (token, head).
+// First, once per token and head and in place: unit vectors over q and k (or the scaled q), decays
+// over a, beta over b.  One wave per (token, key head) and per (token, head).
+enum ScanKind : int { SCAN_CHANNEL_DELTA = 0, SCAN_HEAD_DELTA = 1, SCAN_DECAYED_OUTER = 2 };
+
 __global__ __launch_bounds__(PI_WAVE) void delta_prepare_kernel(float* __restrict__ qkv, long qkv_stride, float* __restrict__ a,
                                                                long a_stride, const float* __restrict__ dt_bias,
                                                                const float* __restrict__ A_log, float* __restrict__ b,
-                                                               long b_stride, int H, int G, int d, float q_scale, float unit_eps) {
+                                                               long b_stride, int H, int G, int d, float q_scale, float unit_eps,
+                                                               int kind, float inv_tau) {
   const long t = blockIdx.x;
   const int j = blockIdx.y, lane = threadIdx.x;
   if (j < G) {
     float* q = qkv + t * qkv_stride + (long)j * d;
+    if (kind == SCAN_DECAYED_OUTER) {
+      for (int c = lane; c < d; c += PI_WAVE) q[c] *= q_scale;
+      return;
+    }
     float* k = q + (long)G * d;
     float q2 = 0.f, k2 = 0.f;
     for (int c = lane; c < d; c += PI_WAVE) {
@@ -378,7 +391,20 @@ __global__ __launch_bounds__(PI_WAVE) void delta_prepare_kernel(float* __restric
     return;
   }
   const int h = j - G;
+  if (kind == SCAN_DECAYED_OUTER) {
+    // sigmoid(z)^(1 / tau) = exp(-softplus(-z) / tau)
+    float* ar = a + t * a_stride + (long)h * d;
+    for (int c = lane; c < d; c += PI_WAVE) ar[c] = expf(-softplus_f(-(ar[c] + dt_bias[(long)h * d + c])) * inv_tau);
+    return;
+  }
   const float A = expf(A_log[h]);
+  if (kind == SCAN_HEAD_DELTA) {
+    if (lane == 0) {
+      a[t * a_stride + h] = expf(-A * softplus_f(a[t * a_stride + h] + dt_bias[h]));
+      b[t * b_stride + h] = sigmoid_f(b[t * b_stride + h]);
+    }
+    return;
+  }
   float* ar = a + t * a_stride + (long)h * d;
   for (int c = lane; c < d; c += PI_WAVE) ar[c] = expf(-A * softplus_f(ar[c] + dt_bias[(long)h * d + c]));
   if (lane == 0) b[t * b_stride + h] = sigmoid_f(b[t * b_stride + h]);
@@ -386,7 +412,7 @@ __global__ __launch_bounds__(PI_WAVE) void delta_prepare_kernel(float* __restric
 
 // Then the walk: q^, k^ and v from qkv, decays from a, beta from b.  A column of S never meets another
 // column, so a wave walks its four columns alone.
-template <int NR, bool SHORT>
+template <int NR, bool SHORT, int KIND>
 __global__ __launch_bounds__((PI_SCAN_WAVES + 1) * PI_WAVE) void delta_scan_kernel(
     float* __restrict__ o, long o_stride, const float* __restrict__ qkv, long qkv_stride, const float* __restrict__ decay,
     long decay_stride, const float* __restrict__ beta, long beta_stride, const int* __restrict__ q_start,
@@ -394,8 +420,8 @@ __global__ __launch_bounds__((PI_SCAN_WAVES + 1) * PI_WAVE) void delta_scan_kern
   constexpr int W = ScanShape<NR, SHORT>::W, CH = ScanShape<NR, SHORT>::CH;
   __shared__ __attribute__((aligned(16))) float sq[2][CH * W];
   __shared__ __attribute__((aligned(16))) float sk[2][CH * W];
-  __shared__ __attribute__((aligned(16))) float sg[2][CH * W];
-  __shared__ float sv[2][CH][PI_SCAN_COLUMNS], sbeta[2][CH];
+  __shared__ __attribute__((aligned(16))) float sg[2][KIND == SCAN_HEAD_DELTA ? 4 : CH * W];
+  __shared__ float sv[2][CH][PI_SCAN_COLUMNS], sbeta[2][CH], sdecay[2][CH];
   const int r = blockIdx.x, h = blockIdx.y, z = blockIdx.z;
   const int wave = threadIdx.x / PI_WAVE, lane = threadIdx.x % PI_WAVE, part = lane % 16;
   const int g = h / (H / G);
@@ -410,7 +436,8 @@ __global__ __launch_bounds__((PI_SCAN_WAVES + 1) * PI_WAVE) void delta_scan_kern
     StagedVectors<W, CH> qs_, ks_, gs_;
     qs_.fetch(src + q_col, qkv_stride, cn, d, (vec & 1) != 0, lane);
     ks_.fetch(src + k_col, qkv_stride, cn, d, (vec & 1) != 0, lane);
-    gs_.fetch(decay + (long)(qs + t0) * decay_stride + (long)h * d, decay_stride, cn, d, (vec & 2) != 0, lane);
+    if constexpr (KIND != SCAN_HEAD_DELTA)
+      gs_.fetch(decay + (long)(qs + t0) * decay_stride + (long)h * d, decay_stride, cn, d, (vec & 2) != 0, lane);
     constexpr int XI = (CH * PI_SCAN_COLUMNS + PI_WAVE - 1) / PI_WAVE;
     float vs[XI];
 #pragma unroll
@@ -418,16 +445,21 @@ __global__ __launch_bounds__((PI_SCAN_WAVES + 1) * PI_WAVE) void delta_scan_kern
       const int i = lane + j * PI_WAVE, tt = i / PI_SCAN_COLUMNS, cc = i % PI_SCAN_COLUMNS;
       vs[j] = (tt < cn && z * PI_SCAN_COLUMNS + cc < dv) ? src[tt * qkv_stride + v_col + cc] : 0.f;
     }
-    const float bt = lane < cn ? beta[(long)(qs + t0 + lane) * beta_stride + h] : 0.f;
+    float bt = 0.f, dc = 0.f;
+    if constexpr (KIND != SCAN_DECAYED_OUTER) bt = lane < cn ? beta[(long)(qs + t0 + lane) * beta_stride + h] : 0.f;
+    if constexpr (KIND == SCAN_HEAD_DELTA) dc = lane < cn ? decay[(long)(qs + t0 + lane) * decay_stride + h] : 0.f;
     qs_.store(sq[buf], lane);
     ks_.store(sk[buf], lane);
-    gs_.store(sg[buf], lane);
+    if constexpr (KIND != SCAN_HEAD_DELTA) gs_.store(sg[buf], lane);
 #pragma unroll
     for (int j = 0; j < XI; ++j) {
       const int i = lane + j * PI_WAVE;
       if (i < CH * PI_SCAN_COLUMNS) (&sv[buf][0][0])[i] = vs[j];
     }
-    if (lane < CH) sbeta[buf][lane] = bt;
+    if (lane < CH) {
+      sbeta[buf][lane] = bt;
+      sdecay[buf][lane] = dc;
+    }
   };
 
   float s[NR];
@@ -451,15 +483,33 @@ __global__ __launch_bounds__((PI_SCAN_WAVES + 1) * PI_WAVE) void delta_scan_kern
       for (int tt = 0; tt < cn; ++tt) {
         const float* qv = &sq[buf][tt * W + part * NR];
         const float* kv = &sk[buf][tt * W + part * NR];
-        const float* gv = &sg[buf][tt * W + part * NR];
-        float d0 = 0.f, d1 = 0.f;
+        float u;
+        if constexpr (KIND == SCAN_DECAYED_OUTER) {
+          const float* gv = &sg[buf][tt * W + part * NR];
 #pragma unroll
-        for (int i = 0; i < NR; ++i) {
-          s[i] *= gv[i];
-          if (i & 1) d1 = fmaf(s[i], kv[i], d1);
-          else d0 = fmaf(s[i], kv[i], d0);
+          for (int i = 0; i < NR; ++i) s[i] *= gv[i];
+          u = sv[buf][tt][cw];
+        } else {
+          float d0 = 0.f, d1 = 0.f;
+          if constexpr (KIND == SCAN_HEAD_DELTA) {
+            const float g1 = sdecay[buf][tt];
+#pragma unroll
+            for (int i = 0; i < NR; ++i) {
+              s[i] *= g1;
+              if (i & 1) d1 = fmaf(s[i], kv[i], d1);
+              else d0 = fmaf(s[i], kv[i], d0);
+            }
+          } else {
+            const float* gv = &sg[buf][tt * W + part * NR];
+#pragma unroll
+            for (int i = 0; i < NR; ++i) {
+              s[i] *= gv[i];
+              if (i & 1) d1 = fmaf(s[i], kv[i], d1);
+              else d0 = fmaf(s[i], kv[i], d0);
+            }
+          }
+          u = sbeta[buf][tt] * (sv[buf][tt][cw] - row16_sum(d0 + d1));
         }
-        const float u = sbeta[buf][tt] * (sv[buf][tt][cw] - row16_sum(d0 + d1));
         float a0 = 0.f, a1 = 0.f;
 #pragma unroll
         for (int i = 0; i < NR; ++i) {
@@ -479,26 +529,37 @@ __global__ __launch_bounds__((PI_SCAN_WAVES + 1) * PI_WAVE) void delta_scan_kern
   }
 }
 
-// qkv, a and b are changed in place (unit vectors, decays, beta); o gets the read-outs.
+// qkv, a and b are changed in place (unit vectors or scaled queries, decays, beta); o gets the read-outs.
+// kind: a ScanKind.  SCAN_HEAD_DELTA: a is [T, H] and dt_bias [H].  SCAN_DECAYED_OUTER: b is not read, A_log neither,
+// unit_eps neither; tau is the root taken of the sigmoid.
 extern "C" int pi_delta_scan(float* o, long o_stride, float* qkv, long qkv_stride, float* a, long a_stride,
                              const float* dt_bias, const float* A_log, float* b, long b_stride, const int* q_start,
                              const int* slots, int R, int T, int longest, float* state, long state_stride, int H, int G, int d, int dv,
-                             float q_scale, float unit_eps, hipStream_t stream) {
-  PI_REQUIRE(H > 0 && H <= 32767 && G > 0 && H % G == 0 && d > 0 && dv > 0, "delta rule: bad sizes heads=%d kv_heads=%d dim=%d vdim=%d", H, G, d, dv);
+                             float q_scale, float unit_eps, int kind, float tau, hipStream_t stream) {
+  PI_REQUIRE(H > 0 && H <= 32767 && G > 0 && H % G == 0 && d > 0 && dv > 0, "state walk: bad sizes heads=%d kv_heads=%d dim=%d vdim=%d", H, G, d, dv);
+  PI_REQUIRE(kind >= SCAN_CHANNEL_DELTA && kind <= SCAN_DECAYED_OUTER, "state walk: unknown kind %d", kind);
+  PI_REQUIRE(kind != SCAN_DECAYED_OUTER || tau > 0.f, "state walk: the decay's root %g must be positive", (double)tau);
+  PI_REQUIRE(kind == SCAN_DECAYED_OUTER || (b && A_log), "state walk: the delta rule needs beta and decay rates");
   const int nr = scan_rows_per_lane(d);
-  PI_REQUIRE(nr > 0, "delta rule: keys of %d channels are more than 256", d);
-  PI_REQUIRE(R >= 0 && T >= 0 && state_stride >= pi_scan_state_floats(H, d, dv), "delta rule: a state row of %ld floats cannot hold %d x %d x %d", state_stride, H, d, dv);
+  PI_REQUIRE(nr > 0, "state walk: keys of %d channels are more than 256", d);
+  PI_REQUIRE(R >= 0 && T >= 0 && state_stride >= pi_scan_state_floats(H, d, dv), "state walk: a state row of %ld floats cannot hold %d x %d x %d", state_stride, H, d, dv);
   if (R == 0 || T == 0) return 0;
   hipLaunchKernelGGL(delta_prepare_kernel, dim3(T, G + H), dim3(PI_WAVE), 0, stream, qkv, qkv_stride, a, a_stride, dt_bias, A_log, b,
-                     b_stride, H, G, d, q_scale, unit_eps);
+                     b_stride, H, G, d, q_scale, unit_eps, kind, kind == SCAN_DECAYED_OUTER ? 1.0f / tau : 0.f);
   if (pi_check_launch("delta_prepare")) return -1;
   // bit 0: q and k may be fetched 16 bytes at a time; bit 1: the decays too
   const int vec = (d % 4 == 0 && qkv_stride % 4 == 0 && (uintptr_t)qkv % 16 == 0 ? 1 : 0) |
                   (d % 4 == 0 && a_stride % 4 == 0 && (uintptr_t)a % 16 == 0 ? 2 : 0);
   const dim3 grid(R, H, (dv + PI_SCAN_COLUMNS - 1) / PI_SCAN_COLUMNS), block((PI_SCAN_WAVES + 1) * PI_WAVE);
-#define PI_LAUNCH_DELTA1(NR_, SHORT_)                                                                                                   \
-  hipLaunchKernelGGL((delta_scan_kernel<NR_, SHORT_>), grid, block, 0, stream, o, o_stride, qkv, qkv_stride, a, a_stride, b, b_stride, \
+#define PI_LAUNCH_DELTA2(NR_, SHORT_, KIND_)                                                                                                   \
+  hipLaunchKernelGGL((delta_scan_kernel<NR_, SHORT_, KIND_>), grid, block, 0, stream, o, o_stride, qkv, qkv_stride, a, a_stride, b, b_stride, \
                      q_start, slots, state, state_stride, H, G, d, dv, vec)
+#define PI_LAUNCH_DELTA1(NR_, SHORT_)                                            \
+  do {                                                                           \
+    if (kind == SCAN_HEAD_DELTA) PI_LAUNCH_DELTA2(NR_, SHORT_, SCAN_HEAD_DELTA); \
+    else if (kind == SCAN_DECAYED_OUTER) PI_LAUNCH_DELTA2(NR_, SHORT_, SCAN_DECAYED_OUTER); \
+    else PI_LAUNCH_DELTA2(NR_, SHORT_, SCAN_CHANNEL_DELTA);                      \
+  } while (0)
 #define PI_LAUNCH_DELTA(NR_) do { if (longest <= 2) PI_LAUNCH_DELTA1(NR_, true); else PI_LAUNCH_DELTA1(NR_, false); } while (0)
   switch (nr) {
     case 1: PI_LAUNCH_DELTA(1); break;
@@ -509,5 +570,6 @@ extern "C" int pi_delta_scan(float* o, long o_stride, float* qkv, long qkv_strid
   }
 #undef PI_LAUNCH_DELTA
 #undef PI_LAUNCH_DELTA1
+#undef PI_LAUNCH_DELTA2
   return pi_check_launch("delta_scan");
 }

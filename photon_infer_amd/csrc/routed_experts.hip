@@ -7,7 +7,11 @@
 //   experts form `groups` equal groups of neighbours, a group's score is its largest s, and
 //   only experts of the `keep` best groups may be chosen (groups <= 1: all may);
 //   the `top` allowed experts with the largest s are chosen, weights = their s (as they are,
-//   or divided by their sum when `renorm`).  Equal scores: the lower index wins.
+//   or divided by their sum + renorm_eps when `renorm`).  Equal scores: the lower index wins.
+//   With a `correction` [E] the choice (of groups and of experts) goes by s + correction; the
+//   weights stay the scores themselves.
+// Experts from `num_real` on are identity experts: they have no matrices, make no tiles, and the
+// weighted sum takes the token's own activations for them.
 #include "common.h"
 
 #define RE_MAX_EXPERTS 1024
@@ -27,8 +31,10 @@ __device__ inline void wave_argmax(float& v, int& idx) {
 }
 
 __global__ __launch_bounds__(PI_WAVE) void route_kernel(int* __restrict__ ids, float* __restrict__ weights, const float* __restrict__ logits,
-                                                        long logits_stride, int E, int top, int groups, int keep, int renorm) {
+                                                        long logits_stride, int E, int top, int groups, int keep, int renorm,
+                                                        const float* __restrict__ correction, float renorm_eps) {
   __shared__ float s[RE_MAX_EXPERTS];
+  __shared__ float c[RE_MAX_EXPERTS];      // what the choice goes by
   __shared__ unsigned char allowed[RE_MAX_EXPERTS];
   __shared__ float gscore[RE_MAX_EXPERTS];
   const long t = blockIdx.x;
@@ -47,6 +53,7 @@ __global__ __launch_bounds__(PI_WAVE) void route_kernel(int* __restrict__ ids, f
   const float inv = 1.0f / sum;
   for (int e = lane; e < E; e += PI_WAVE) {
     s[e] *= inv;
+    c[e] = correction ? s[e] + correction[e] : s[e];
     allowed[e] = (groups <= 1) ? 1 : 0;
   }
   __syncthreads();
@@ -54,7 +61,7 @@ __global__ __launch_bounds__(PI_WAVE) void route_kernel(int* __restrict__ ids, f
     const int per = E / groups;
     for (int g = lane; g < groups; g += PI_WAVE) {
       float best = -INFINITY;
-      for (int e = g * per; e < (g + 1) * per; ++e) best = fmaxf(best, s[e]);
+      for (int e = g * per; e < (g + 1) * per; ++e) best = fmaxf(best, c[e]);
       gscore[g] = best;
     }
     __syncthreads();
@@ -79,16 +86,17 @@ __global__ __launch_bounds__(PI_WAVE) void route_kernel(int* __restrict__ ids, f
     float v = -INFINITY;
     int idx = 0x7fffffff;
     for (int e = lane; e < E; e += PI_WAVE)
-      if (allowed[e] && s[e] > v) {
-        v = s[e];
+      if (allowed[e] && c[e] > v) {
+        v = c[e];
         idx = e;
       }
     wave_argmax(v, idx);
     if (idx >= E) {          // fewer allowed experts than choices: the entry counts nothing
       idx = 0;
       v = 0.f;
-    } else if (lane == 0) {
-      allowed[idx] = 0;
+    } else {
+      v = s[idx];
+      if (lane == 0) allowed[idx] = 0;
     }
     wsum += v;
     if (lane == 0) {
@@ -98,19 +106,19 @@ __global__ __launch_bounds__(PI_WAVE) void route_kernel(int* __restrict__ ids, f
     __syncthreads();
   }
   if (renorm && lane == 0) {
-    const float r = 1.0f / wsum;
+    const float r = 1.0f / (wsum + renorm_eps);
     for (int j = 0; j < top; ++j) weights[t * top + j] *= r;
   }
 }
 
 extern "C" int pi_route(int* ids, float* weights, const float* logits, long logits_stride, int T, int E, int top, int groups,
-                        int keep, int renorm, hipStream_t stream) {
+                        int keep, int renorm, const float* correction, float renorm_eps, hipStream_t stream) {
   PI_REQUIRE(T >= 0 && E > 0 && E <= RE_MAX_EXPERTS, "routing: %d experts (at most %d)", E, RE_MAX_EXPERTS);
   PI_REQUIRE(top > 0 && top <= E, "routing: %d choices among %d experts", top, E);
   PI_REQUIRE(groups <= 1 || (E % groups == 0 && keep > 0 && keep <= groups), "routing: %d experts in %d groups, %d kept", E, groups, keep);
   PI_REQUIRE(groups <= 1 || (long)keep * (E / groups) >= top, "routing: %d kept groups of %d experts hold fewer than %d choices", keep, groups > 0 ? E / groups : 0, top);
   if (T == 0) return 0;
-  hipLaunchKernelGGL(route_kernel, dim3(T), dim3(PI_WAVE), 0, stream, ids, weights, logits, logits_stride, E, top, groups, keep, renorm);
+  hipLaunchKernelGGL(route_kernel, dim3(T), dim3(PI_WAVE), 0, stream, ids, weights, logits, logits_stride, E, top, groups, keep, renorm, correction, renorm_eps);
   return pi_check_launch("route");
 }
 
@@ -119,6 +127,8 @@ extern "C" int pi_route(int* ids, float* weights, const float* logits, long logi
 //   row_entry[row] = entry, entry_row[entry] = row (entries of one expert keep their order),
 //   tiles of up to `tile` rows that never straddle two experts: tile_expert[i] (-1: unused),
 //   tile_row0[i], tile_rows[i]; max_tiles = ceil(N / tile) + E bounds their number.
+// Entries whose id is not in 0 .. E - 1 (identity experts) own no row: their entry_row is 0, and the rows
+// that stay empty behind the last expert's name entry 0, so that whoever walks all N rows stays in bounds.
 // One block of 1024 threads; wave w places the experts w, w + 16, ...
 __global__ __launch_bounds__(1024) void group_entries_kernel(const int* __restrict__ ids, int N, int E, int* __restrict__ row_entry,
                                                              int* __restrict__ entry_row, int* __restrict__ tile_expert,
@@ -147,6 +157,9 @@ __global__ __launch_bounds__(1024) void group_entries_kernel(const int* __restri
     tstart[E] = tacc;
   }
   __syncthreads();
+  for (int i = start[E] + tid; i < N; i += 1024) row_entry[i] = 0;
+  for (int i = tid; i < N; i += 1024)
+    if (ids[i] < 0 || ids[i] >= E) entry_row[i] = 0;
   for (int i = tstart[E] + tid; i < max_tiles; i += 1024) {
     tile_expert[i] = -1;
     tile_row0[i] = 0;
@@ -286,22 +299,36 @@ extern "C" int pi_grouped_gemm_general(void* C, int c_dtype, long ldc, const voi
   return pi_check_launch("grouped_gemm_general");
 }
 
-// out[t, :] (+)= sum_j weights[t, j] * y[entry_row[t * top + j], :], choices in order (float32)
+// out[t, :] (+)= sum_j weights[t, j] * y[entry_row[t * top + j], :], choices in order (float32); a choice whose
+// id is num_real or more (ids given) stands for the token's own activations h[t, :] instead
+template <typename TH>
 __global__ void combine_choices_kernel(float* __restrict__ out, const float* __restrict__ y, const float* __restrict__ weights,
-                                       const int* __restrict__ entry_row, int top, int D, int accumulate) {
+                                       const int* __restrict__ entry_row, int top, int D, int accumulate, const int* __restrict__ ids,
+                                       int num_real, const TH* __restrict__ h) {
   const long t = blockIdx.x;
   const int d = blockIdx.y * blockDim.x + threadIdx.x;
   if (d >= D) return;
   float acc = 0.f;
-  for (int j = 0; j < top; ++j) acc = fmaf(weights[t * top + j], y[(long)entry_row[t * top + j] * D + d], acc);
+  for (int j = 0; j < top; ++j) {
+    const bool own = ids && ids[t * top + j] >= num_real;
+    const float v = own ? to_float(h[t * D + d]) : y[(long)entry_row[t * top + j] * D + d];
+    acc = fmaf(weights[t * top + j], v, acc);
+  }
   out[t * D + d] = accumulate ? out[t * D + d] + acc : acc;
 }
 
 extern "C" int pi_combine_choices(float* out, const float* y, const float* weights, const int* entry_row, int T, int top, int D,
-                                  int accumulate, hipStream_t stream) {
+                                  int accumulate, const int* ids, int num_real, const void* h, int h_dtype, hipStream_t stream) {
   PI_REQUIRE(T >= 0 && top > 0 && D > 0, "combine: bad sizes");
+  PI_REQUIRE(!ids || h, "combine: identity experts need the tokens' activations");
   if (T == 0) return 0;
   PI_REQUIRE((D + 255) / 256 <= 65535, "combine: rows of %d are too long", D);
-  hipLaunchKernelGGL(combine_choices_kernel, dim3(T, (D + 255) / 256), dim3(256), 0, stream, out, y, weights, entry_row, top, D, accumulate);
+  const dim3 grid(T, (D + 255) / 256), block(256);
+  if (ids && h_dtype == PI_BF16)
+    hipLaunchKernelGGL(combine_choices_kernel<bf16_t>, grid, block, 0, stream, out, y, weights, entry_row, top, D, accumulate, ids, num_real, (const bf16_t*)h);
+  else if (!ids || h_dtype == PI_F32)
+    hipLaunchKernelGGL(combine_choices_kernel<float>, grid, block, 0, stream, out, y, weights, entry_row, top, D, accumulate, ids, num_real, (const float*)h);
+  else
+    return pi_fail("combine: unsupported activation dtype %d", h_dtype);
   return pi_check_launch("combine_choices");
 }

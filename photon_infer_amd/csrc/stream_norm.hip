@@ -154,6 +154,163 @@ extern "C" int pi_branch_norm_add(float* x, void* h, int h_dtype, const float* a
   return pi_check_launch("branch_norm_add");
 }
 
+// ---------------------------------------------------------------- layer norm with weight and bias
+// LN(v; w, b) = (v - mean) / sqrt(mean of squared deviations + eps) * w + b, all float32.  The row sits in
+// LDS between the passes: the mean first, then the deviations' squares, so that nothing is cancelled.
+__device__ inline void layer_norm_stats(const float* row, int D, float eps, float* scratch, float& mean, float& rinv) {
+  float s = 0.f;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) s += row[d];
+  mean = block_sum(s, scratch) / D;
+  float q = 0.f;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    const float dev = row[d] - mean;
+    q = fmaf(dev, dev, q);
+  }
+  rinv = 1.0f / sqrtf(block_sum(q, scratch) / D + eps);
+}
+
+// out[m, :] = LN(x[rows[m] or m, :]; w, b) in the activation type
+template <typename TO>
+__global__ __launch_bounds__(256) void layer_norm_kernel(TO* __restrict__ out, const float* __restrict__ x, const int* __restrict__ rows,
+                                                         const float* __restrict__ w, const float* __restrict__ b, float eps, int D,
+                                                         int x_rows) {
+  extern __shared__ float row[];
+  __shared__ float scratch[16];
+  const long m = blockIdx.x;
+  const long r = rows ? rows[m] : m;
+  const bool ok = r >= 0 && r < x_rows;          // a row outside the stream gives NaN, no fault
+  for (int d = threadIdx.x; d < D; d += blockDim.x) row[d] = ok ? x[r * D + d] : NAN;
+  __syncthreads();
+  float mean, rinv;
+  layer_norm_stats(row, D, eps, scratch, mean, rinv);
+  for (int d = threadIdx.x; d < D; d += blockDim.x) out[m * D + d] = from_float<TO>((row[d] - mean) * rinv * w[d] + b[d]);
+}
+
+extern "C" int pi_layer_norm(void* out, int out_dtype, const float* x, const int* rows, const float* w, const float* b, float eps,
+                             int M, int D, int x_rows, hipStream_t stream) {
+  PI_REQUIRE(M >= 0 && D > 0 && D <= 16000 && x_rows >= 0, "layer norm: bad sizes M=%d D=%d", M, D);
+  PI_REQUIRE(out && x && w && b, "layer norm: output, input, weight and bias are needed");
+  if (M == 0) return 0;
+  const int threads = D >= 1024 ? 256 : (D >= 256 ? 128 : 64);
+  const size_t lds = (size_t)D * sizeof(float);
+  if (out_dtype == PI_F32)
+    hipLaunchKernelGGL(layer_norm_kernel<float>, dim3(M), dim3(threads), lds, stream, (float*)out, x, rows, w, b, eps, D, x_rows);
+  else if (out_dtype == PI_BF16)
+    hipLaunchKernelGGL(layer_norm_kernel<bf16_t>, dim3(M), dim3(threads), lds, stream, (bf16_t*)out, x, rows, w, b, eps, D, x_rows);
+  else
+    return pi_fail("layer norm: unsupported dtype %d", out_dtype);
+  return pi_check_launch("layer_norm");
+}
+
+// A sublayer's result joins the stream through a layer norm, and the next sublayer's input is made on the way:
+//   y = a (+ a_bias)                                                      (one branch)
+//   y = (rms(a (+ a_bias); wa) + rms(b; wb)) / 2                           (two branches side by side)
+//   x <- x + LN(y; pw, pb);   h = LN(x; nw, nb)   (nw null: no h)
+// with rms(v; w) = v / sqrt(mean(v^2) + eps) * w.  One block per token; the row stays in LDS throughout.
+template <typename TH>
+__global__ __launch_bounds__(256) void sandwich_norm_add_kernel(float* __restrict__ x, TH* __restrict__ h, const float* __restrict__ a,
+                                                                const float* __restrict__ a_bias, const float* __restrict__ wa,
+                                                                const float* __restrict__ b, const float* __restrict__ wb,
+                                                                const float* __restrict__ pw, const float* __restrict__ pb,
+                                                                const float* __restrict__ nw, const float* __restrict__ nb, float eps,
+                                                                int D) {
+  extern __shared__ float row[];
+  __shared__ float scratch[32];
+  const long t = blockIdx.x;
+  const float* ar = a + t * D;
+  const float* br = b ? b + t * D : nullptr;
+  if (wa) {
+    float sa = 0.f, sb = 0.f;
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+      const float va = ar[d] + (a_bias ? a_bias[d] : 0.f);
+      row[d] = va;
+      sa = fmaf(va, va, sa);
+      if (br) {
+        const float vb = br[d];
+        sb = fmaf(vb, vb, sb);
+      }
+    }
+    block_sum2(sa, sb, scratch);
+    const float ra = 1.0f / sqrtf(sa / D + eps), rb = br ? 1.0f / sqrtf(sb / D + eps) : 0.f;
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+      float v = row[d] * ra * wa[d];
+      if (br) v = 0.5f * (v + br[d] * rb * wb[d]);
+      row[d] = v;
+    }
+  } else {
+    for (int d = threadIdx.x; d < D; d += blockDim.x) row[d] = ar[d] + (a_bias ? a_bias[d] : 0.f);
+  }
+  __syncthreads();
+  float mean, rinv;
+  layer_norm_stats(row, D, eps, scratch, mean, rinv);
+  float* xr = x + t * D;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    const float v = xr[d] + ((row[d] - mean) * rinv * pw[d] + pb[d]);
+    xr[d] = v;
+    row[d] = v;
+  }
+  if (!nw) return;
+  __syncthreads();
+  layer_norm_stats(row, D, eps, scratch, mean, rinv);
+  for (int d = threadIdx.x; d < D; d += blockDim.x) h[t * D + d] = from_float<TH>((row[d] - mean) * rinv * nw[d] + nb[d]);
+}
+
+extern "C" int pi_sandwich_norm_add(float* x, void* h, int h_dtype, const float* a, const float* a_bias, const float* wa,
+                                    const float* b, const float* wb, const float* pw, const float* pb, const float* nw,
+                                    const float* nb, float eps, int T, int D, hipStream_t stream) {
+  PI_REQUIRE(T >= 0 && D > 0 && D <= 16000, "norm and add: bad sizes T=%d D=%d", T, D);
+  PI_REQUIRE(x && a && pw && pb, "norm and add: the stream, a result and the norm's weight and bias are needed");
+  PI_REQUIRE(!b || (wa && wb), "norm and add: two branches need both their weights");
+  PI_REQUIRE(!nw || (nb && h), "norm and add: the next norm needs its bias and a place for its result");
+  if (T == 0) return 0;
+  const int threads = D >= 1024 ? 256 : (D >= 256 ? 128 : 64);
+  const size_t lds = (size_t)D * sizeof(float);
+  if (!nw || h_dtype == PI_F32)
+    hipLaunchKernelGGL(sandwich_norm_add_kernel<float>, dim3(T), dim3(threads), lds, stream, x, (float*)h, a, a_bias, wa, b, wb, pw, pb, nw, nb, eps, D);
+  else if (h_dtype == PI_BF16)
+    hipLaunchKernelGGL(sandwich_norm_add_kernel<bf16_t>, dim3(T), dim3(threads), lds, stream, x, (bf16_t*)h, a, a_bias, wa, b, wb, pw, pb, nw, nb, eps, D);
+  else
+    return pi_fail("norm and add: unsupported activation dtype %d", h_dtype);
+  return pi_check_launch("sandwich_norm_add");
+}
+
+// ---------------------------------------------------------------- two attention maps into one head
+// Differential attention: head n of kv group g holds the results a1 and a2 of two softmax maps over the same
+// values.  In `attn` the maps are heads of their own, ordered [g][map][head within group] (so that the
+// attention kernels see map m of group g as kv head 2 g + m).  out[t, n, :] = mult * o / sqrt(mean(o^2) + eps),
+// o = a1 - lam * a2, float32; one wave per (token, head).
+template <typename TO, typename TI>
+__global__ __launch_bounds__(PI_WAVE) void diff_combine_kernel(TO* __restrict__ out, const TI* __restrict__ attn, float lam, float eps,
+                                                               float mult, int H, int G, int dv) {
+  const long t = blockIdx.x;
+  const int n = blockIdx.y, lane = threadIdx.x;
+  const int per = H / G, g = n / per, i = n % per;
+  const TI* a1 = attn + (t * 2 * H + (long)(2 * g) * per + i) * dv;
+  const TI* a2 = a1 + (long)per * dv;
+  float ss = 0.f;
+  for (int c = lane; c < dv; c += PI_WAVE) {
+    const float o = fmaf(-lam, to_float(a2[c]), to_float(a1[c]));
+    ss = fmaf(o, o, ss);
+  }
+  const float r = mult / sqrtf(wave_sum(ss) / dv + eps);
+  for (int c = lane; c < dv; c += PI_WAVE)
+    out[(t * H + n) * dv + c] = from_float<TO>(fmaf(-lam, to_float(a2[c]), to_float(a1[c])) * r);
+}
+
+extern "C" int pi_diff_combine(void* out, int out_dtype, const void* attn, int in_dtype, float lam, float eps, float mult, int T, int H,
+                               int G, int dv, hipStream_t stream) {
+  PI_REQUIRE(T >= 0 && H > 0 && H <= 65535 && G > 0 && H % G == 0 && dv > 0, "two maps: bad sizes heads=%d kv_heads=%d vdim=%d", H, G, dv);
+  if (T == 0) return 0;
+  const dim3 grid(T, H), block(PI_WAVE);
+#define DC_GO(TO, TI) hipLaunchKernelGGL((diff_combine_kernel<TO, TI>), grid, block, 0, stream, (TO*)out, (const TI*)attn, lam, eps, mult, H, G, dv)
+  if (out_dtype == PI_F32 && in_dtype == PI_F32) DC_GO(float, float);
+  else if (out_dtype == PI_BF16 && in_dtype == PI_BF16) DC_GO(bf16_t, bf16_t);
+  else if (out_dtype == PI_BF16 && in_dtype == PI_F32) DC_GO(bf16_t, float);
+  else return pi_fail("two maps: unsupported dtypes out=%d in=%d", out_dtype, in_dtype);
+#undef DC_GO
+  return pi_check_launch("diff_combine");
+}
+
 template <typename TO>
 __global__ void cast_stream_kernel(TO* __restrict__ out, const float* __restrict__ x, long n) {
   const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;

@@ -1,2 +1,2 @@
 """Architectures the engine ships; importing this package registers them."""
-from . import dafidra, dokanex, llama, rorevik  # noqa: F401
+from . import dafidra, dokanex, llama, muretar, rorevik  # noqa: F401

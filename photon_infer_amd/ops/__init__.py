@@ -324,7 +324,7 @@ def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
                   req_of_token: torch.Tensor, rotary, num_heads: int, num_kv_heads: int, head_dim: int,
                   k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
                   block_table: Optional[torch.Tensor], page_size: int, pieces=None, write_kv: Optional[bool] = None,
-                  value_dim: Optional[int] = None) -> None:
+                  value_dim: Optional[int] = None, bias: Optional[torch.Tensor] = None) -> None:
     """Rotate q in place by each token's position; rotate k and store k, v into the pages.
     ``value_dim``: the width of a value head when it differs from ``head_dim``.
 
@@ -334,10 +334,17 @@ def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
     ``pieces``: the q|k|v projection still split over k (``fast.Partials`` with columns
     [q heads | k heads | v heads]); then ``q`` is the output buffer for the rotated queries and
     ``k``/``v`` are not given (``write_kv`` says whether the cache is written).
+    ``bias``: float32, one per column of the projection [q heads | k heads | v heads]; it is added in float32 before
+    the rotation (with ``pieces``: to their sum, so the biased projection is never held in reduced precision).
     """
-    _gpu(q, k, v, positions, req_of_token, k_cache, v_cache, block_table)
+    _gpu(q, k, v, positions, req_of_token, k_cache, v_cache, block_table, bias)
     T = q.shape[0]
     vd = head_dim if value_dim is None else int(value_dim)
+    if bias is not None:
+        with_kv = bool(write_kv) if pieces is not None else k is not None
+        need = num_heads * head_dim + (num_kv_heads * (head_dim + vd) if with_kv else 0)
+        if bias.dtype != torch.float32 or not bias.is_contiguous() or bias.numel() < need:
+            raise KernelError(f"rope: the projection's bias must be contiguous float32 with at least {need} entries")
     if value_dim is None:
         check_attention_sizes(num_heads, num_kv_heads, head_dim)
     else:
@@ -357,11 +364,11 @@ def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
             _ptr(req_of_token) if write else None, table_ptr, rdim, int(bool(inter)), T, num_heads, num_kv_heads,
             head_dim, int(write), _ptr(k_cache) if write else None, _ptr(v_cache) if write else None,
             _ptr(block_table) if write else None, block_table.shape[1] if write else 0, page_size if write else 0, pages,
-            pieces.part.data_ptr(), pieces.splits, pieces.N, 0, q_size, q_size + kv_size, vd, _stream())
+            pieces.part.data_ptr(), pieces.splits, pieces.N, 0, q_size, q_size + kv_size, vd, _ptr(bias), _stream())
         return
     write = k is not None
     table_ptr, rdim, inter, _keep = _rotary_args(rotary, positions, T)
-    if not write and rdim == 0:
+    if not write and rdim == 0 and bias is None:
         return
     pages = 0
     if write:
@@ -377,7 +384,8 @@ def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
         _rows(v, "v") if write else 0, _dt(q), positions.data_ptr(), _ptr(req_of_token) if write else None,
         table_ptr, rdim, int(bool(inter)), T, num_heads, num_kv_heads, head_dim, int(write),
         _ptr(k_cache) if write else None, _ptr(v_cache) if write else None, _ptr(block_table) if write else None,
-        block_table.shape[1] if write else 0, page_size if write else 0, pages, None, 0, 0, 0, 0, 0, vd, _stream())
+        block_table.shape[1] if write else 0, page_size if write else 0, pages, None, 0, 0, 0,
+        num_heads * head_dim, num_heads * head_dim + num_kv_heads * head_dim, vd, _ptr(bias), _stream())
 
 
 def decode_attention_from_projection(out: torch.Tensor, qkv, ctx, rotary, num_heads: int, num_kv_heads: int,
@@ -548,6 +556,93 @@ def cast_stream(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     out = torch.empty(x.shape, dtype=dtype, device=x.device)
     _lib.call("core", "pi_cast_stream", out.data_ptr(), _dt(out), x.data_ptr(), x.numel(), _stream())
     return out
+
+
+def layer_norm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float,
+               rows: Optional[torch.Tensor] = None) -> None:
+    """out[m, :] = (x[r, :] - mean) / sqrt(mean of squared deviations + eps) * weight + bias, r = rows[m] (or m);
+    ``x`` float32, weight and bias float32, everything computed in float32 and rounded once into ``out``."""
+    _gpu(out, x, weight, bias, rows)
+    M, D = out.shape
+    if x.dtype != torch.float32 or not x.is_contiguous() or x.dim() != 2 or x.shape[1] != D or not out.is_contiguous():
+        raise KernelError(f"layer norm: input must be contiguous float32 [*, {D}], got {x.dtype} {tuple(x.shape)}")
+    _f32_vector(weight, D, "layer norm weight")
+    _f32_vector(bias, D, "layer norm bias")
+    if rows is None:
+        if x.shape[0] != M:
+            raise KernelError(f"layer norm: {x.shape[0]} input rows for {M} output rows")
+    else:
+        _i32(rows, "layer norm rows", M)
+    _lib.call("core", "pi_layer_norm", out.data_ptr(), _dt(out), x.data_ptr(), _ptr(rows), weight.data_ptr(), bias.data_ptr(),
+              float(eps), M, D, x.shape[0], _stream())
+
+
+def sandwich_norm_add(x: torch.Tensor, a: torch.Tensor, post, eps: float, nxt=None, h_dtype: Optional[torch.dtype] = None,
+                      w_a: Optional[torch.Tensor] = None, b: Optional[torch.Tensor] = None, w_b: Optional[torch.Tensor] = None,
+                      a_bias: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """x += LN(y; post) with y = a (+ a_bias), or rms(a (+ a_bias); w_a), or the mean of rms(a (+ a_bias); w_a) and
+    rms(b; w_b); LN the layer norm with (weight, bias) = ``post``, rms(v; w) = v / sqrt(mean(v^2) + eps) * w; all
+    float32.  With ``nxt`` = (weight, bias) the layer norm of the new stream is returned in ``h_dtype`` (what the next
+    sublayer reads), made in the same pass."""
+    _gpu(x, a, b, w_a, w_b, a_bias)
+    T, D = x.shape
+    for t, what in ((x, "stream"), (a, "result"), (b, "second result")):
+        if t is not None and (t.dtype != torch.float32 or not t.is_contiguous() or tuple(t.shape) != (T, D)):
+            raise KernelError(f"norm and add: the {what} must be contiguous float32 [{T}, {D}]")
+    vectors = [(post[0], "norm weight"), (post[1], "norm bias"), (w_a, "branch weight"), (w_b, "second branch weight"), (a_bias, "result bias")]
+    if nxt is not None:
+        vectors += [(nxt[0], "next norm weight"), (nxt[1], "next norm bias")]
+    for t, what in vectors:
+        _f32_vector(t, D, f"norm and add {what}")
+    h = None
+    if nxt is not None:
+        h = torch.empty((T, D), dtype=h_dtype or torch.float32, device=x.device)
+    _lib.call("core", "pi_sandwich_norm_add", x.data_ptr(), _ptr(h), _dt(h) if h is not None else PI_F32, a.data_ptr(), _ptr(a_bias),
+              _ptr(w_a), _ptr(b), _ptr(w_b), post[0].data_ptr(), post[1].data_ptr(), _ptr(nxt[0]) if nxt is not None else None,
+              _ptr(nxt[1]) if nxt is not None else None, float(eps), T, D, _stream())
+    return h
+
+
+def diff_combine(out: torch.Tensor, attn: torch.Tensor, lam: float, eps: float, mult: float, heads: int, kv_heads: int,
+                 value_dim: int) -> None:
+    """Two attention maps per head into one result: ``attn`` [T, 2 * heads * value_dim] holds the maps as heads of
+    their own in the order [kv group][map][head within the group]; out[t, n, :] = mult * o / sqrt(mean(o^2) + eps) with
+    o = map 1 - lam * map 2 of head n, float32 arithmetic."""
+    _gpu(out, attn)
+    T = out.shape[0]
+    if tuple(out.shape) != (T, heads * value_dim) or tuple(attn.shape) != (T, 2 * heads * value_dim) or not (out.is_contiguous() and attn.is_contiguous()):
+        raise KernelError(f"two maps: expected contiguous [{T}, {2 * heads * value_dim}] -> [{T}, {heads * value_dim}], got {tuple(attn.shape)} -> {tuple(out.shape)}")
+    _lib.call("core", "pi_diff_combine", out.data_ptr(), _dt(out), attn.data_ptr(), _dt(attn), float(lam), float(eps), float(mult), T,
+              int(heads), int(kv_heads), int(value_dim), _stream())
+
+
+EPI_RELU2 = 5        # the matrix-core products' epilogue: max(c, 0)^2 rounded to bfloat16
+
+
+def gemm_relu_squared(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, ws: Optional[KernelWorkspace] = None) -> None:
+    """out[M, N] = max(a @ w^T, 0)^2, the square taken on the product's float32 result.  With bfloat16 operands and more
+    rows than the weight-streaming products take, product and activation are one kernel."""
+    _gpu(out, a, w)
+    M, N = out.shape
+    if w.shape[0] != N or a.shape != (M, w.shape[1]):
+        raise KernelError(f"gemm_relu_squared: shapes do not agree: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
+    if M == 0:
+        return
+    if _FAST and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and out.is_contiguous():
+        from . import fast
+        if fast.gemm_relu_squared(out, a, w, M, N, a.shape[1], _rows(a, "gemm a"), _rows(w, "gemm w")):
+            return
+    u = torch.empty((M, N), dtype=torch.float32, device=a.device)
+    gemm(u, a, w, ws=ws)
+    relu_squared(out, u)
+
+
+def relu_squared(out: torch.Tensor, a: torch.Tensor) -> None:
+    """out = max(a, 0)^2 from float32 ``a`` into ``out`` (any type), squared before the one rounding."""
+    _gpu(out, a)
+    if a.dtype != torch.float32 or out.shape != a.shape or not (a.is_contiguous() and out.is_contiguous()):
+        raise KernelError("squared relu: expected a contiguous float32 input and an output of its shape")
+    _lib.call("core", "pi_relu_squared", out.data_ptr(), _dt(out), a.data_ptr(), a.numel(), _stream())
 
 
 def branch_norm_add(x: torch.Tensor, a: torch.Tensor, w_outer: torch.Tensor, eps: float, mult: float,
@@ -747,8 +842,11 @@ def matrix_memory_scan(out: torch.Tensor, proj: torch.Tensor, offsets, i_bias: t
 
 
 def head_norm_gate(y: torch.Tensor, o: torch.Tensor, gates: torch.Tensor, weight: torch.Tensor, eps: float, heads: int, value_dim: int,
-                   mult: float = 1.0) -> None:
-    """y[t, h, :] = mult * o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * weight[h, :] * sigmoid(gates[t, h, :])."""
+                   mult: float = 1.0, gate: str = "sigmoid") -> None:
+    """y[t, h, :] = mult * o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * weight[h, :] * act(gates[t, h, :]), ``gate``
+    naming act: "sigmoid", or "silu" (z * sigmoid(z))."""
+    if gate not in ("sigmoid", "silu"):
+        raise KernelError(f"head norm: gate activation '{gate}' is not known (sigmoid, silu)")
     _gpu(y, o, gates, weight)
     T, N = y.shape[0], heads * value_dim
     if tuple(y.shape) != (T, N) or not y.is_contiguous():
@@ -758,23 +856,26 @@ def head_norm_gate(y: torch.Tensor, o: torch.Tensor, gates: torch.Tensor, weight
             raise KernelError(f"head norm: {what} must be float32 [{T}, >= {N}]")
     _f32_vector(weight, N, "head norm weight")
     _lib.call("core", "pi_head_norm_gate", y.data_ptr(), _dt(y), o.data_ptr(), _rows(o, "o"), gates.data_ptr(), _rows(gates, "gates"),
-              weight.data_ptr(), float(eps), T, heads, value_dim, float(mult), _stream())
+              weight.data_ptr(), float(eps), T, heads, value_dim, float(mult), int(gate == "silu"), _stream())
 
 
 # ----------------------------------------------------------------------------- routed experts
-def route(logits: torch.Tensor, top: int, groups: int = 1, keep: int = 1, renorm: bool = False):
+def route(logits: torch.Tensor, top: int, groups: int = 1, keep: int = 1, renorm: bool = False,
+          correction: Optional[torch.Tensor] = None, renorm_eps: float = 0.0):
     """Choose ``top`` experts per row of float32 router logits: (ids int32 [T, top], weights float32
     [T, top]).  Scores are the softmax over all experts; with ``groups`` > 1 only experts of the
     ``keep`` groups with the largest best score may be chosen; weights are the chosen scores
-    (divided by their sum when ``renorm``)."""
-    _gpu(logits)
+    (divided by their sum + ``renorm_eps`` when ``renorm``).  ``correction`` (float32 [E]): the choice goes
+    by score + correction, the weights by the scores alone."""
+    _gpu(logits, correction)
     T, E = logits.shape
+    _f32_vector(correction, E, "routing correction")
     if logits.dtype != torch.float32:
         raise KernelError("routing: logits must be float32")
     ids = torch.empty((T, top), dtype=torch.int32, device=logits.device)
     weights = torch.empty((T, top), dtype=torch.float32, device=logits.device)
     _lib.call("core", "pi_route", ids.data_ptr(), weights.data_ptr(), logits.data_ptr(), _rows(logits, "router logits"), T, E,
-              int(top), int(groups), int(keep), int(bool(renorm)), _stream())
+              int(top), int(groups), int(keep), int(bool(renorm)), _ptr(correction), float(renorm_eps), _stream())
     return ids, weights
 
 
@@ -800,7 +901,8 @@ def grouped_tile_rows(dtype: torch.dtype) -> int:
 
 
 def group_entries(ids: torch.Tensor, num_experts: int, tile: Optional[int] = None) -> ExpertRows:
-    """Sort the entries of ``ids`` (int32 [T, top]) by expert, on the device."""
+    """Sort the entries of ``ids`` (int32 [T, top]) by expert, on the device.  Entries whose id is ``num_experts``
+    or more (identity experts) get no row and no tile."""
     _gpu(ids)
     _i32(ids, "expert ids")
     N = ids.numel()
@@ -873,16 +975,38 @@ def grouped_gemm_swiglu(out: torch.Tensor, a: torch.Tensor, w_gate_up: torch.Ten
     swiglu(out, gu, block)
 
 
-def combine_choices(out: torch.Tensor, y: torch.Tensor, weights: torch.Tensor, rows: ExpertRows, accumulate: bool = False) -> None:
-    """out[t] (+)= sum over the token's choices of weight * y[row of (t, choice)], in choice order (float32)."""
-    _gpu(out, y, weights)
+def grouped_gemm_relu_squared(out: torch.Tensor, a: torch.Tensor, w_up: torch.Tensor, rows: ExpertRows) -> None:
+    """out[row] = max(a[row] @ W^T, 0)^2 with the row's expert's matrix; ``w_up`` is [experts, F, K].  The square is taken on
+    the product's float32 result."""
+    _gpu(out, a, w_up)
+    if out.shape != (rows.rows, w_up.shape[1]):
+        raise KernelError(f"grouped squared relu: out {tuple(out.shape)} does not match {rows.rows} x {w_up.shape[1]}")
+    if rows.rows == 0:
+        return
+    if out.dtype == torch.bfloat16 and out.is_contiguous() and _grouped_fast(out, a, w_up, rows, EPI_RELU2):
+        return
+    u = torch.empty((rows.rows, w_up.shape[1]), dtype=torch.float32, device=a.device)
+    grouped_gemm(u, a, w_up, rows)
+    relu_squared(out, u)
+
+
+def combine_choices(out: torch.Tensor, y: torch.Tensor, weights: torch.Tensor, rows: ExpertRows, accumulate: bool = False,
+                    ids: Optional[torch.Tensor] = None, num_real: int = 0, h: Optional[torch.Tensor] = None) -> None:
+    """out[t] (+)= sum over the token's choices of weight * y[row of (t, choice)], in choice order (float32).
+    With ``ids`` (int32 [T, top]), ``num_real`` and the tokens' activations ``h`` [T, D]: a choice whose id is
+    ``num_real`` or more is an identity expert and contributes weight * h[t]."""
+    _gpu(out, y, weights, ids, h)
+    if ids is not None:
+        _i32(ids, "expert ids", weights.numel())
+        if h is None or h.shape != out.shape or not h.is_contiguous():
+            raise KernelError("combine: identity experts need the tokens' activations, contiguous and as wide as the output")
     T, D = out.shape
     if out.dtype != torch.float32 or y.dtype != torch.float32 or not (out.is_contiguous() and y.is_contiguous()) or y.shape != (rows.rows, D):
         raise KernelError(f"combine: expected float32 out [{T}, {D}] and y [{rows.rows}, {D}]")
     if weights.dtype != torch.float32 or not weights.is_contiguous() or weights.numel() != rows.rows:
         raise KernelError("combine: one float32 weight per entry is needed")
     _lib.call("core", "pi_combine_choices", out.data_ptr(), y.data_ptr(), weights.data_ptr(), rows.entry_row.data_ptr(), T, rows.top, D,
-              int(bool(accumulate)), _stream())
+              int(bool(accumulate)), _ptr(ids), int(num_real), _ptr(h), _dt(h) if h is not None else PI_F32, _stream())
 
 
 # ----------------------------------------------------------------------------- mixers with a state of fixed size
@@ -985,9 +1109,12 @@ def gated_group_norm(out: torch.Tensor, y: torch.Tensor, z: torch.Tensor, weight
               float(eps), float(mult), T, N, int(parts), _stream())
 
 
-def delta_scan(o: torch.Tensor, qkv: torch.Tensor, a: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, b: torch.Tensor,
-               ctx, state: torch.Tensor, heads: int, kv_heads: int, key_dim: int, value_dim: int, q_scale: float,
-               unit_eps: float) -> None:
+SCAN_KINDS = {"channel_delta": 0, "head_delta": 1, "decayed_outer": 2}
+
+
+def delta_scan(o: torch.Tensor, qkv: torch.Tensor, a: torch.Tensor, dt_bias: torch.Tensor, a_log: Optional[torch.Tensor],
+               b: Optional[torch.Tensor], ctx, state: torch.Tensor, heads: int, kv_heads: int, key_dim: int, value_dim: int,
+               q_scale: float, unit_eps: float, kind: str = "channel_delta", tau: float = 1.0) -> None:
     """The gated delta rule with a decay per head and key channel over the step's tokens, from and
     into the requests' state rows (``state`` float32 [slots, >= scan_state_floats(heads, key_dim, value_dim)]):
     ``S <- diag(decay) S; u = beta (v - S^T k^); S <- S + k^ u^T; o = S^T q^`` with unit vectors
@@ -995,21 +1122,32 @@ def delta_scan(o: torch.Tensor, qkv: torch.Tensor, a: torch.Tensor, dt_bias: tor
     ``beta = sigmoid(b)``.  ``qkv``, ``a`` and ``b`` are CHANGED IN PLACE: a first kernel turns them into the unit
     vectors, the decays and beta, once per token and head, before the walk reads them.  ``qkv`` float32 rows hold q and k [kv_heads * key_dim each] and v
     [heads * value_dim]; ``a`` float32 [T, heads * key_dim]; ``b`` float32 [T, heads] (a column view
-    is fine); ``o`` float32 [T, heads * value_dim]."""
+    is fine); ``o`` float32 [T, heads * value_dim].
+
+    ``kind`` "head_delta": the same with one decay per head, ``S <- decay S``: ``a`` is [T, heads] and ``dt_bias`` [heads].
+    ``kind`` "decayed_outer" (gated linear attention): ``S <- diag(decay) S + k v^T; o = S^T (q * q_scale)`` with
+    ``decay = sigmoid(a + dt_bias)^(1 / tau)`` per head and key channel; no unit vectors, no ``b``, no ``a_log``."""
+    if kind not in SCAN_KINDS:
+        raise KernelError(f"state walk: kind '{kind}' is not known ({', '.join(SCAN_KINDS)})")
     _gpu(o, qkv, a, dt_bias, a_log, b, state)
     T = o.shape[0]
+    per_head = kind == "head_delta"
+    outer = kind == "decayed_outer"
     ldo = _f32_rows(o, T, heads * value_dim, "delta rule output")
     ldq = _f32_rows(qkv, T, 2 * kv_heads * key_dim + heads * value_dim, "delta rule input")
-    lda = _f32_rows(a, T, heads * key_dim, "delta rule decays")
-    ldb = _f32_rows(b, T, heads, "delta rule beta")
-    _f32_vector(dt_bias, heads * key_dim, "delta rule decay bias")
-    _f32_vector(a_log, heads, "delta rule decay rate")
+    lda = _f32_rows(a, T, heads if per_head else heads * key_dim, "delta rule decays")
+    ldb = 0 if outer else _f32_rows(b, T, heads, "delta rule beta")
+    _f32_vector(dt_bias, heads if per_head else heads * key_dim, "delta rule decay bias")
+    if not outer:
+        _f32_vector(a_log, heads, "delta rule decay rate")
+    elif not tau > 0.0:
+        raise KernelError(f"state walk: the root taken of the decays must be positive, got {tau}")
     _state_rows(state, scan_state_floats(heads, key_dim, value_dim), "delta rule")
     _i32(ctx.q_start, "q_start", ctx.R + 1)
     _i32(ctx.slots, "slots", ctx.R)
-    _lib.call("core", "pi_delta_scan", o.data_ptr(), ldo, qkv.data_ptr(), ldq, a.data_ptr(), lda, dt_bias.data_ptr(), a_log.data_ptr(),
-              b.data_ptr(), ldb, ctx.q_start.data_ptr(), ctx.slots.data_ptr(), ctx.R, T, int(getattr(ctx, "max_q_len", 0) or T), state.data_ptr(), state.stride(0), heads,
-              kv_heads, key_dim, value_dim, float(q_scale), float(unit_eps), _stream())
+    _lib.call("core", "pi_delta_scan", o.data_ptr(), ldo, qkv.data_ptr(), ldq, a.data_ptr(), lda, dt_bias.data_ptr(), _ptr(a_log),
+              _ptr(b), ldb, ctx.q_start.data_ptr(), ctx.slots.data_ptr(), ctx.R, T, int(getattr(ctx, "max_q_len", 0) or T), state.data_ptr(), state.stride(0), heads,
+              kv_heads, key_dim, value_dim, float(q_scale), float(unit_eps), SCAN_KINDS[kind], float(tau), _stream())
 
 
 def clamped_glu(out: torch.Tensor, gate_up: torch.Tensor, gate_bias: torch.Tensor, up_bias: Optional[torch.Tensor], limit: float,

@@ -22,10 +22,10 @@ _SIGNATURES = {
         "pi_causal_conv_silu": [P, L, P, L, P, P, I, I, I, P, P, I, I, P, L, P],
         "pi_state_space_scan": [P, L, P, L, P, L, P, P, P, P, P, I, I, P, L, I, I, I, I, P],
         "pi_gated_group_norm": [P, I, L, P, L, P, L, P, F, F, I, I, I, P],
-        "pi_delta_scan": [P, L, P, L, P, L, P, P, P, L, P, P, I, I, I, P, L, I, I, I, I, F, F, P],
+        "pi_delta_scan": [P, L, P, L, P, L, P, P, P, L, P, P, I, I, I, P, L, I, I, I, I, F, F, I, F, P],
         "pi_rmsnorm": [P, I, P, P, P, I, F, I, I, P, I, L, P],
         "pi_swiglu": [P, P, I, I, I, I, P],
-        "pi_rope_kv_write": [P, L, P, L, P, L, I, P, P, P, I, I, I, I, I, I, I, P, P, P, I, I, L, P, I, I, I, I, I, I, P],
+        "pi_rope_kv_write": [P, L, P, L, P, L, I, P, P, P, I, I, I, I, I, I, I, P, P, P, I, I, L, P, I, I, I, I, I, I, P, P],
         "pi_gemm_general": [P, I, L, P, I, L, P, I, L, I, I, I, I, P],
         "pi_paged_attention_general": [P, L, P, L, P, P, I, P, I, P, P, I, I, I, I, I, F, I, L, I, P, L, I, P, P, P, F, F, I, P],
         "pi_branch_norm_add": [P, P, I, P, P, P, P, P, F, F, I, I, P],
@@ -34,12 +34,16 @@ _SIGNATURES = {
         "pi_latent_kv_write": [P, L, I, P, L, P, P, P, P, P, F, I, I, I, I, I, P, P, P, I, I, L, P, I, L, P],
         "pi_head_gemm": [P, L, I, P, L, I, P, I, I, I, I, I, I, P, I, P],
         "pi_matrix_memory_scan": [P, L, P, L, I, I, I, I, I, P, P, F, F, P, P, I, P, L, I, I, I, I, I, I, P, L, P],
-        "pi_head_norm_gate": [P, I, P, L, P, L, P, F, I, I, I, F, P],
-        "pi_route": [P, P, P, L, I, I, I, I, I, I, P],
+        "pi_head_norm_gate": [P, I, P, L, P, L, P, F, I, I, I, F, I, P],
+        "pi_route": [P, P, P, L, I, I, I, I, I, I, P, F, P],
         "pi_group_entries": [P, I, I, P, P, P, P, P, I, I, P],
         "pi_gather_rows": [P, P, I, P, I, I, I, P],
         "pi_grouped_gemm_general": [P, I, L, P, I, L, P, I, L, L, P, P, P, I, I, I, P],
-        "pi_combine_choices": [P, P, P, P, I, I, I, I, P],
+        "pi_combine_choices": [P, P, P, P, I, I, I, I, P, I, P, I, P],
+        "pi_relu_squared": [P, I, P, L, P],
+        "pi_layer_norm": [P, I, P, P, P, P, F, I, I, I, P],
+        "pi_sandwich_norm_add": [P, P, I, P, P, P, P, P, P, P, P, P, F, I, I, P],
+        "pi_diff_combine": [P, I, P, I, F, F, F, I, I, I, I, P],
         "pi_paged_attention_general_ranges": [I, I, I],
         "pi_rope_table": [P, P, P, I, I, F, P],
         "pi_sample": [P, P, L, P, P, I, I, P, L, P],

@@ -27,6 +27,7 @@ from . import _lib
 from .workspace import GEMM_PART_FLOATS, KernelWorkspace, KeyRanges, Partials, PendingUpdate
 
 EPI_BF16, EPI_F32, EPI_ACCUM, EPI_SWIGLU = 0, 1, 2, 3
+EPI_RELU2 = 5
 SKINNY_MAX_ROWS = 128          # up to this many tokens the weight-streaming kernels serve a product (measured against the tile kernel)
 ROWS_PER_BLOCK = 32            # weight rows per block of the skinny kernel
 BLOCKS_PER_UNIT = 2            # blocks of it wanted per compute unit to keep HBM busy (measured: 512 on 256 units; 384 and 768 are slower)
@@ -278,6 +279,16 @@ def gemm_pieces(a, w, ws: Optional[KernelWorkspace]) -> Optional[Partials]:
     if splits <= 1:
         return None
     return _skinny(0, EPI_F32, N, a, w, M, N, K, lda, ldw, splits, ws)
+
+
+def gemm_relu_squared(out, a, w, M, N, K, lda, ldw) -> bool:
+    """out [M, N] bfloat16 = max(a @ w^T, 0)^2 as the tile product's epilogue; only for more rows than the
+    weight-streaming products take (those have no such epilogue)."""
+    if not _gemm_ok(a, w, K, lda, ldw) or M <= SKINNY_MAX_ROWS:
+        return False
+    _lib.call("bf16", "pi_gemm_mfma", out.data_ptr(), EPI_RELU2, out.stride(0), a.data_ptr(), lda, w.data_ptr(), ldw, M, N, K, 1,
+              _stream())
+    return True
 
 
 def gemm_swiglu(out, a, w, M, N, K, lda, ldw, ws: Optional[KernelWorkspace] = None) -> bool:

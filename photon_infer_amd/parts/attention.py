@@ -18,7 +18,10 @@ Further options, each a constructor parameter: values of another width than keys
 (``value_dim``), a cap on the scores (``softcap`` c: the scaled score s becomes
 ``c * tanh(s / c)`` before the softmax), a factor on the mixer's result (``out_scale``, for
 arrangements that weigh mixers side by side; applied to the attention's float32 output before
-its one rounding, so that the output projection needs no second pass), and other tensor names.
+its one rounding, so that the output projection needs no second pass), other tensor names, biases on the
+q, k and v projections (``qkv_bias``) and on the output projection (``o_bias``; tensor names with ``bias_suffix``
+added; added in float32, the first three before the rotation), and ``accumulate`` False: the result is written into the
+tensor handed to ``forward`` instead of added to it.
 """
 from __future__ import annotations
 
@@ -28,6 +31,7 @@ from typing import Dict, List, Optional
 import torch
 
 from .. import ops
+from ..errors import UnsupportedModelError
 from ..weights.loader import TensorSpec
 from .base import MIXERS, PAGE, KVCacheSpec, LayerCache, Mixer, PagedCacheSpec, PagedTensor, PositionEncoding, StepContext
 
@@ -51,6 +55,11 @@ class PagedAttention(Mixer):
         out_scale: float = 1.0,
         names=("q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight"),
         any_head_size: bool = False,
+        qkv_bias: bool = False,
+        o_bias: bool = False,
+        bias_suffix: str = ".b",
+        accumulate: bool = True,
+        bias_to_caller: bool = False,
     ):
         self.hidden_size = int(hidden_size)
         self.num_heads = int(num_heads)
@@ -64,6 +73,11 @@ class PagedAttention(Mixer):
         self.softcap = float(softcap) if softcap else 0.0
         self.out_scale = float(out_scale)
         self.names = tuple(names)          # the q, k, v and o matrices' names after the part's prefix
+        self.qkv_bias, self.o_bias, self.bias_suffix, self.accumulate = bool(qkv_bias), bool(o_bias), bias_suffix, bool(accumulate)
+        # True: the output projection's bias is not added here; whoever called reads it from ``pending_bias``
+        # and adds it in a pass of its own (an arrangement that normalises the result anyway)
+        self.bias_to_caller = bool(bias_to_caller) and self.o_bias
+        self.pending_bias: Optional[torch.Tensor] = None
         self.q_size = self.num_heads * self.head_dim
         self.kv_size = self.num_kv_heads * self.head_dim
         self.v_size = self.num_kv_heads * self.value_dim
@@ -85,6 +99,11 @@ class PagedAttention(Mixer):
                 TensorSpec(self.names[2], (self.v_size, self.hidden_size)),
             ]
         specs.append(TensorSpec(self.names[3], (self.hidden_size, self.o_size)))
+        if self.qkv_bias:
+            sizes = [self.q_size] + ([self.kv_size, self.v_size] if self.own_kv else [])
+            specs += [TensorSpec(n + self.bias_suffix, (size,), "small_bias") for n, size in zip(self.names, sizes)]
+        if self.o_bias:
+            specs.append(TensorSpec(self.names[3] + self.bias_suffix, (self.hidden_size,), "small_bias"))
         if self.position is not None:     # a position encoding with tensors of its own keeps them under "position."
             specs += [s.with_prefix(POSITION_PREFIX) for s in self.position.tensor_specs()]
         return specs
@@ -116,6 +135,12 @@ class PagedAttention(Mixer):
         common = torch.float32 if any(m.dtype == torch.float32 for m in mats) else mats[0].dtype
         self.w_qkv = torch.cat([m.to(common) for m in mats], dim=0).contiguous()
         self.w_o = tensors[self.names[3]]
+        self.b_qkv = self.b_o = None
+        if self.qkv_bias:
+            self.b_qkv = torch.cat([tensors[n + self.bias_suffix].to(torch.float32) for n in self.names[:len(mats)]]).contiguous()
+        if self.o_bias:
+            self.b_o = tensors[self.names[3] + self.bias_suffix].to(torch.float32).contiguous()
+            self.pending_bias = self.b_o if self.bias_to_caller else None
         if self.position is not None:
             own = {n[len(POSITION_PREFIX):]: t for n, t in tensors.items() if n.startswith(POSITION_PREFIX)}
             self.position.load(own, dtype, device)
@@ -130,8 +155,17 @@ class PagedAttention(Mixer):
         fused_position = self.position is None or rotary is not None
         table = ctx.block_tables[cache.group]
         ws = ctx.workspace
-        qkv = ops.qkv_projection(h, self.w_qkv, self.dtype, ws) if fused_position else None
-        if qkv is not None and ctx.all_decode and not self.with_options:
+        if self.qkv_bias:
+            if not fused_position:
+                raise UnsupportedModelError("biased projections go with a rotation (or none), not with another position encoding")
+            # float32 results (a tensor, or the pieces of a product split over k) so that the biased projection is
+            # rounded once, after the rotation
+            qkv = ops.qkv_projection(h, self.w_qkv, torch.float32, ws)
+            if isinstance(qkv, torch.Tensor):
+                qkv = ops.Partials(qkv.view(1, T, qkv.shape[1]), 1, T, qkv.shape[1])
+        else:
+            qkv = ops.qkv_projection(h, self.w_qkv, self.dtype, ws) if fused_position else None
+        if qkv is not None and ctx.all_decode and not self.with_options and not self.qkv_bias:
             # single tokens only: one kernel rotates, writes the cache and attends
             attn = torch.empty((T, self.q_size), dtype=self.dtype, device=h.device)
             done = ops.decode_attention_from_projection(attn, qkv, ctx, rotary, self.num_heads, self.num_kv_heads,
@@ -140,14 +174,17 @@ class PagedAttention(Mixer):
                                                         leave_ranges=self.w_o.numel() * self.w_o.element_size())
             if done:
                 # the output, or its key ranges still to be merged, which the product does as it reads them
-                ops.gemm(x, done if isinstance(done, ops.KeyRanges) else attn, self.w_o, accumulate=True, may_defer=getattr(ctx, "may_defer", False), ws=ws)
+                ops.gemm(x, done if isinstance(done, ops.KeyRanges) else attn, self.w_o, accumulate=self.accumulate,
+                         may_defer=self.accumulate and not self.o_bias and getattr(ctx, "may_defer", False), ws=ws)
+                if self.o_bias and not self.bias_to_caller:
+                    ops.add_row_bias(x, self.b_o)
                 return
         if qkv is not None and not isinstance(qkv, torch.Tensor):
             # the projection is still in pieces (split over k): the rotation kernel sums them
             q = torch.empty((T, self.q_size), dtype=self.dtype, device=h.device)
             ops.rope_kv_write(q, None, None, ctx.positions, ctx.req_of_token, rotary, self.num_heads,
                               self.num_kv_heads, self.head_dim, cache.k, cache.v, table, cache.page_size,
-                              pieces=qkv, write_kv=writes, value_dim=self.value_dim)
+                              pieces=qkv, write_kv=writes, value_dim=self.value_dim, bias=self.b_qkv)
         else:
             if qkv is None:
                 qkv = torch.empty((T, self.w_qkv.shape[0]), dtype=self.dtype, device=h.device)
@@ -174,7 +211,10 @@ class PagedAttention(Mixer):
                 self.scale, self.window or 0, ws,
             )
         # where the arrangement allows it, the product stays in pieces for the stream's next reader
-        ops.gemm(x, attn, self.w_o, accumulate=True, may_defer=getattr(ctx, "may_defer", False), ws=ws)
+        ops.gemm(x, attn, self.w_o, accumulate=self.accumulate,
+                 may_defer=self.accumulate and not self.o_bias and getattr(ctx, "may_defer", False), ws=ws)
+        if self.o_bias and not self.bias_to_caller:
+            ops.add_row_bias(x, self.b_o)
 
 
 MIXERS.register("attention", PagedAttention)

@@ -197,3 +197,87 @@ class OutputNormBlock(Block):
 
 
 BLOCKS.register("output_norm", OutputNormBlock)
+
+
+class SandwichBlock(Block):
+    """A norm in front of every sublayer and another behind it:
+
+        x <- x + post1(mix(pre1(x)));   x <- x + post2(ffn(pre2(x)))     (no feed-forward: the first only)
+
+    ``mix`` is one mixer, or two side by side that read the same input: then each result is first RMS-normalised
+    over the width with a weight of its own and the two are averaged.  The four norms are layer norms with weight and
+    bias (``LayerNorm``).  The branch norms, the mean, the norm behind the sublayer, the add and the norm in front of the
+    next sublayer of the block are one kernel.  The mixers and the feed-forward write their result
+    (``accumulate=False``) instead of adding it.
+
+    ``branches``: [(prefix, mixer, (prefix, rmsnorm) or None)]; ``pre1`` / ``post1`` / ``pre2`` / ``post2`` / ``ffn``: (prefix, part).
+    """
+
+    reads_deferred = False
+
+    def __init__(self, branches, pre1: Tuple[str, Norm], post1: Tuple[str, Norm], pre2=None, post2=None, ffn=None):
+        if not 1 <= len(branches) <= 2:
+            raise UnsupportedModelError(f"a sandwich block holds one mixer or two side by side, not {len(branches)}")
+        if len(branches) == 2 and any(b[2] is None for b in branches):
+            raise UnsupportedModelError("two mixers side by side each need the norm of their result")
+        if not ((ffn is None) == (pre2 is None) == (post2 is None)):
+            raise UnsupportedModelError("a feed-forward and its two norms come together")
+        self.branches = list(branches)
+        self.pre1, self.post1 = pre1[1], post1[1]
+        self.pre2, self.post2, self.ffn = (pre2[1], post2[1], ffn[1]) if ffn is not None else (None, None, None)
+        self._named: List[Tuple[str, Part]] = [pre1, post1] + [(p, m) for p, m, _ in branches] + [n for _, _, n in branches if n is not None]
+        if ffn is not None:
+            self._named += [pre2, post2, ffn]
+        for _, part in [(p, m) for p, m, _ in branches] + ([ffn] if ffn is not None else []):
+            if getattr(part, "accumulate", True):
+                raise UnsupportedModelError(f"{type(part).__name__} must be built with accumulate=False inside a sandwich block")
+        for n in (self.pre1, self.post1, self.pre2, self.post2):
+            if n is not None and not hasattr(n, "weight_bias_f32"):
+                raise UnsupportedModelError(f"a sandwich block's norms are layer norms with weight and bias, not {type(n).__name__}")
+
+    def mixers(self) -> List[Mixer]:
+        return [m for _, m, _ in self.branches]
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [s.with_prefix(p) for p, part in self._named for s in part.tensor_specs()]
+
+    def load(self, tensors: Dict[str, torch.Tensor], dtype, device) -> None:
+        super().load(tensors, dtype, device)
+        # a part's tensors: those named by its own list (prefixes here may be prefixes of one another)
+        for prefix, part in self._named:
+            names = [prefix + s.name for s in part.tensor_specs()]
+            part.load({n[len(prefix):]: tensors[n] for n in names}, dtype, device)
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(part.graph_safe for _, part in self._named)
+
+    def streamed_weights(self) -> List[torch.Tensor]:
+        return [w for _, part in self._named for w in part.streamed_weights()]
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache) -> None:
+        caches = cache if isinstance(cache, (list, tuple)) else [cache]
+        ctx.may_defer = False
+        h = self.pre1.forward(x, ctx)
+        outs = []
+        for (_, mixer, _), c in zip(self.branches, caches):
+            out = torch.empty_like(x)
+            mixer.forward(h, out, ctx, c)
+            outs.append(out)
+        norms = [n[1] if n is not None else None for _, _, n in self.branches]
+        nxt = self.pre2.weight_bias_f32() if self.ffn is not None else None
+        # a mixer may leave the bias of its last product to this kernel (``pending_bias``)
+        a_bias = getattr(self.branches[0][1], "pending_bias", None)
+        w_a = norms[0].weight_f32() if norms[0] is not None else None
+        if len(outs) == 2:
+            h = ops.sandwich_norm_add(x, outs[0], self.post1.weight_bias_f32(), self.post1.eps, nxt, self.dtype, w_a=w_a, b=outs[1],
+                                      w_b=norms[1].weight_f32(), a_bias=a_bias)
+        else:
+            h = ops.sandwich_norm_add(x, outs[0], self.post1.weight_bias_f32(), self.post1.eps, nxt, self.dtype, w_a=w_a, a_bias=a_bias)
+        if self.ffn is not None:
+            out = torch.empty_like(x)
+            self.ffn.forward(h, out, ctx)
+            ops.sandwich_norm_add(x, out, self.post2.weight_bias_f32(), self.post2.eps)
+
+
+BLOCKS.register("sandwich", SandwichBlock)

@@ -103,3 +103,72 @@ class ChannelDeltaRule(Mixer):
 
 
 MIXERS.register("channel_delta_rule", ChannelDeltaRule)
+
+
+class GatedDeltaRule(Mixer):
+    """The gated delta rule with one decay per head (the paper's own form), full-rank projections for the decay and
+    for a silu output gate:
+
+    * q, k, v as above (convolutions, silu, unit vectors, q times ``key_dim^-1/2``);
+    * ``beta = sigmoid(W_b h)`` and ``decay = exp(-exp(A_log_n) softplus(W_a h + dt_bias_n))``, one each per head;
+    * per head: ``S <- decay S``, ``u = beta (v - S^T k)``, ``S <- S + k u^T``, ``o = S^T q``;
+    * each head's o RMS-normalised over value_dim with the weight ``norm`` (shared by the heads), times
+      ``silu(W_g h)``, then ``W_o``.
+
+    One projection gives everything that is read from h, as float32: rows [q | k | v | b | a | g]."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, key_dim: int, value_dim: int, conv_taps: int, eps: float,
+                 accumulate: bool = True):
+        self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.key_dim, self.value_dim, self.conv_taps = int(key_dim), int(value_dim), int(conv_taps)
+        self.eps, self.accumulate = float(eps), bool(accumulate)
+        if self.num_heads % self.num_kv_heads:
+            raise UnsupportedModelError(f"delta rule: {self.num_heads} heads is not a multiple of {self.num_kv_heads} key heads")
+        if not 1 <= self.conv_taps <= ops.CONV_MAX_TAPS or self.key_dim > 256:
+            raise UnsupportedModelError(f"delta rule: {self.conv_taps} taps (at most {ops.CONV_MAX_TAPS}), keys of {self.key_dim} (at most 256)")
+        self.qk_size, self.v_size = self.num_kv_heads * self.key_dim, self.num_heads * self.value_dim
+        self.channels = 2 * self.qk_size + self.v_size
+        self.conv_floats = (self.conv_taps - 1) * self.channels
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        D, H, t = self.hidden_size, self.num_heads, self.conv_taps
+        return [TensorSpec("q", (self.qk_size, D)), TensorSpec("q.conv", (self.qk_size, t), "taps"),
+                TensorSpec("k", (self.qk_size, D)), TensorSpec("k.conv", (self.qk_size, t), "taps"),
+                TensorSpec("v", (self.v_size, D)), TensorSpec("v.conv", (self.v_size, t), "taps"),
+                TensorSpec("b", (H, D)), TensorSpec("A_log", (H,), "bias"), TensorSpec("norm", (self.value_dim,), "norm"),
+                TensorSpec("a", (H, D)), TensorSpec("dt_bias", (H,), "bias"), TensorSpec("g", (self.v_size, D)),
+                TensorSpec("o", (D, self.v_size))]
+
+    def cache_spec(self):
+        return StateSpec((self.conv_floats + ops.scan_state_floats(self.num_heads, self.key_dim, self.value_dim),), torch.float32)
+
+    def load(self, tensors: Dict[str, torch.Tensor], dtype, device) -> None:
+        super().load(tensors, dtype, device)
+        self.w_in = torch.cat([tensors[n] for n in ("q", "k", "v", "b", "a", "g")], dim=0).contiguous()
+        self.w_o = tensors["o"]
+        self.w_conv = torch.cat([tensors[n] for n in ("q.conv", "k.conv", "v.conv")], dim=0).contiguous()
+        f32 = lambda t: t.to(torch.float32).contiguous()
+        self.dt_bias, self.a_log = f32(tensors["dt_bias"]), f32(tensors["A_log"])
+        self.w_norm = f32(tensors["norm"]).repeat(self.num_heads).contiguous()      # per head, as the norm kernel indexes it
+
+    def streamed_weights(self) -> List[torch.Tensor]:
+        return [self.w_in, self.w_o]
+
+    def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> None:
+        T, ws, C, H = h.shape[0], ctx.workspace, self.channels, self.num_heads
+        f32 = lambda n: torch.empty((T, n), dtype=torch.float32, device=h.device)
+        proj = f32(C + 2 * H + self.v_size)
+        ops.gemm(proj, h, self.w_in, ws=ws)
+        qkv = f32(C)
+        ops.causal_conv_silu(qkv, proj[:, :C], self.w_conv, None, ctx, cache.state[:, :self.conv_floats])
+        o = f32(self.v_size)
+        ops.delta_scan(o, qkv, proj[:, C + H:C + 2 * H], self.dt_bias, self.a_log, proj[:, C:C + H], ctx, cache.state[:, self.conv_floats:],
+                       H, self.num_kv_heads, self.key_dim, self.value_dim, self.key_dim ** -0.5, UNIT_EPS, kind="head_delta")
+        y = torch.empty((T, self.v_size), dtype=self.dtype, device=h.device)
+        ops.head_norm_gate(y, o, proj[:, C + 2 * H:], self.w_norm, self.eps, H, self.value_dim, gate="silu")
+        ops.gemm(x, y, self.w_o, accumulate=self.accumulate, may_defer=self.accumulate and getattr(ctx, "may_defer", False), ws=ws)
+
+
+MIXERS.register("gated_delta_rule", GatedDeltaRule)

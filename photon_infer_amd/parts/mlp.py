@@ -133,3 +133,36 @@ class ClampedGLU(FeedForward):
 
 
 FEED_FORWARDS.register("clamped_glu", ClampedGLU)
+
+
+class SquaredReluMLP(FeedForward):
+    """A feed-forward without a gate: ``y = W_down act(W_up h)`` with ``act(z) = max(z, 0)^2``, no biases.  The square
+    is taken on the product's float32 result, before the one rounding.  ``accumulate`` False: the result is written
+    into the tensor handed to ``forward`` instead of added to it."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, names=("up", "down"), accumulate: bool = True):
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.names, self.accumulate = tuple(names), bool(accumulate)
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        I, D = self.intermediate_size, self.hidden_size
+        return [TensorSpec(self.names[0], (I, D)), TensorSpec(self.names[1], (D, I))]
+
+    def load(self, tensors: Dict[str, torch.Tensor], dtype, device) -> None:
+        super().load(tensors, dtype, device)
+        self.w_up, self.w_down = tensors[self.names[0]], tensors[self.names[1]]
+
+    def streamed_weights(self) -> List[torch.Tensor]:
+        return [self.w_up, self.w_down]
+
+    def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
+        ws = ctx.workspace if ctx is not None else None
+        act = torch.empty((h.shape[0], self.intermediate_size), dtype=self.dtype, device=h.device)
+        ops.gemm_relu_squared(act, h, self.w_up, ws=ws)
+        ops.gemm(x, act, self.w_down, accumulate=self.accumulate,
+                 may_defer=self.accumulate and getattr(ctx, "may_defer", False), ws=ws)
+
+
+FEED_FORWARDS.register("squared_relu_mlp", SquaredReluMLP)

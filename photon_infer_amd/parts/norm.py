@@ -1,4 +1,4 @@
-"""RMS normalisation part.
+"""Normalisation parts: RMS norm, and layer norm with weight and bias.
 
 Formula (include/photon/ops/kernels/rmsnorm_kernel.hpp:55-87): mean of squares over
 the row, ``rms = sqrt(mean + eps)`` with eps inside the root, ``y = w * (x / rms)``;
@@ -53,3 +53,39 @@ class RMSNorm(Norm):
 
 
 NORMS.register("rmsnorm", RMSNorm)
+
+
+class LayerNorm(Norm):
+    """Layer norm with weight and bias: ``(x - mean) / sqrt(variance + eps) * w + b``, the variance the mean of the
+    squared deviations; mean, variance and scaling in float32, rounded once to the compute dtype.
+    ``tensor_name``: the weight's name after the part's prefix (may be empty: the prefix is the name); the bias is
+    that name plus ``bias_suffix``."""
+
+    graph_safe = True
+
+    def __init__(self, dim: int, eps: float, tensor_name: str = "weight", bias_suffix: str = ".b"):
+        self.dim, self.eps = int(dim), float(eps)
+        self.tensor_name, self.bias_name = tensor_name, tensor_name + bias_suffix
+        self.weight: Optional[torch.Tensor] = None
+        self.bias: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [TensorSpec(self.tensor_name, (self.dim,), "norm"), TensorSpec(self.bias_name, (self.dim,), "small_bias")]
+
+    def load(self, tensors: Dict[str, torch.Tensor], dtype, device) -> None:
+        super().load(tensors, dtype, device)
+        self.weight = tensors[self.tensor_name].to(torch.float32).contiguous()
+        self.bias = tensors[self.bias_name].to(torch.float32).contiguous()
+
+    def weight_bias_f32(self):
+        """(weight, bias) as the kernels that fold this norm into another pass take them."""
+        return self.weight, self.bias
+
+    def forward(self, x: torch.Tensor, ctx=None, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        m = x.shape[0] if rows is None else rows.shape[0]
+        out = torch.empty((m, self.dim), dtype=self.dtype, device=x.device)
+        ops.layer_norm(out, x, self.weight, self.bias, self.eps, rows)
+        return out
+
+
+NORMS.register("layernorm", LayerNorm)
