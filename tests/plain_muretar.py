@@ -236,14 +236,24 @@ def route(z: torch.Tensor, correction: torch.Tensor, top: int):
     return order, w / (w.sum() + WEIGHT_SUM_EPS)
 
 
-def routed_experts(h: torch.Tensor, mlp: dict, W: Dict[str, torch.Tensor], p: str, act_round: Round = None, choices: Optional[list] = None) -> torch.Tensor:
-    """``choices``: per token the experts to use instead of the router's own choice (weights still from the scores)."""
+def routed_experts(h: torch.Tensor, mlp: dict, W: Dict[str, torch.Tensor], p: str, act_round: Round = None, choices: Optional[list] = None,
+                   margins: Optional[list] = None, chosen: Optional[list] = None) -> torch.Tensor:
+    """``choices``: per token the experts to use instead of the router's own choice (weights still from the scores).
+    ``chosen`` / ``margins``: lists that receive, per token, the router's own choice and by how much (in choice score) its
+    last chosen expert beat the best one left out."""
     real, ident, top = mlp["router"]["experts"], mlp["router"].get("identity", 0), mlp["router"]["top"]
     T = h.shape[0]
     z = h @ W[p + "router"].T
     out = torch.zeros_like(h)
     for t in range(T):
         order, w = route(z[t], W[p + "correction"], top)
+        if chosen is not None:
+            chosen.append(list(order))
+        if margins is not None:
+            sc = torch.exp(z[t] - z[t].max())
+            sc = sc / sc.sum() + W[p + "correction"]
+            ranked = sorted((float(v) for v in sc), reverse=True)
+            margins.append(ranked[top - 1] - ranked[top] if top < len(ranked) else float("inf"))
         if choices is not None:
             s = torch.exp(z[t] - z[t].max())
             s = s / s.sum()
@@ -263,9 +273,10 @@ def routed_experts(h: torch.Tensor, mlp: dict, W: Dict[str, torch.Tensor], p: st
 
 # ------------------------------------------------------------------ the model
 def forward(config: dict, W: Dict[str, torch.Tensor], tokens: List[int], act_round: Round = None, streams: Optional[list] = None,
-            choices: Optional[dict] = None) -> torch.Tensor:
+            choices: Optional[dict] = None, margins: Optional[dict] = None, chosen: Optional[dict] = None) -> torch.Tensor:
     """Logits [T, vocab] (float64) of the whole sequence.  ``streams``: a list that receives the residual
-    stream after every layer.  ``choices``: {layer index: per token the experts to use}."""
+    stream after every layer.  ``choices``: {layer index: per token the experts to use}; ``margins`` / ``chosen``: dicts
+    that receive, per routed layer, what ``routed_experts`` reports."""
     W = {n: t.to(F64) for n, t in W.items()}
     eps = float(config["norm"]["eps"])
     x = W["embed"][torch.tensor(tokens, dtype=torch.long)]
@@ -292,7 +303,8 @@ def forward(config: dict, W: Dict[str, torch.Tensor], tokens: List[int], act_rou
             if mlp["kind"] == "dense":
                 y = gated_unit(h, W, p + "mlp.", act_round)
             else:
-                y = routed_experts(h, mlp, W, p + "mlp.", act_round, None if choices is None else choices.get(i))
+                y = routed_experts(h, mlp, W, p + "mlp.", act_round, None if choices is None else choices.get(i),
+                                   None if margins is None else margins.setdefault(i, []), None if chosen is None else chosen.setdefault(i, []))
             x = x + ln(y, "norm2b")
         if streams is not None:
             streams.append(x.clone())
