@@ -1,7 +1,7 @@
 #!/usr/bin/python3
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode1b|long1b|serve3b|mixed8b|dafidra|rorevik|dokanex]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode1b|long1b|serve3b|mixed8b|dafidra|rorevik|dokanex|muretar]
                     [--batch 8,1,64] [--context 4096] [--dtype bf16|fp32]
 
 Every workload prints ONE JSON line.  The default, ``decode1b`` (Llama 3.2 1B layer sizes):  ``value`` is decoded tokens per second at batch 8 with the context
@@ -49,6 +49,11 @@ Llama 3.2 1B's and 3B's, beside a Llama of the same width, depth and vocabulary,
 chunks of 1,024 positions with unit heads, capped scores, a sink and a gate, every second such layer on the keys and
 values of the one before; a tied, capped head) at layer sizes like Llama 3.2 1B's and 3B's, beside a Llama of the same
 width, depth and vocabulary, measured the same way.
+
+``--workload muretar``: the Muretar design (layer norms around every sublayer; gated linear attention, differential
+attention, rotary attention with biases beside a gated delta rule; dense and routed feed-forwards with identity and shared
+experts) at layer sizes like Llama 3.2 1B's and 3B's, beside a Llama of the same width, depth and vocabulary, measured the
+same way.
 
 Weights are random (N(0, 0.02), norms 1), token ids uniform random; no dataset is involved.
 """
@@ -665,6 +670,79 @@ def workload_dokanex(args) -> int:
     return 0
 
 
+def muretar_config(width, heads, kv_heads, head_dim, ff, vocab, layers):
+    """A Muretar of Llama-like layer sizes, layers in fours: gated linear attention (heads of 128 keys and 256 values, as
+    wide as the model in its values, a decay projection through 16, tau 16) with a dense gated feed-forward; the same with
+    routed experts; differential attention (half the Llama's heads with two maps each, values twice as wide as keys) with
+    routed experts; attention as the Llama's (with biases, frequencies divided by 2) beside a gated delta rule (heads of 128
+    keys and values, half as many key heads, four taps) with routed experts.  Routed feed-forwards: 16 experts of a quarter of
+    the dense width and 2 identity experts, 4 per token, a shared expert of the same width."""
+    gla = dict(heads=width // 256, dim=128, vdim=256, tau=16.0, decay_rank=16)
+    diff = dict(heads=heads // 2, kv_heads=max(1, kv_heads // 2), dim=head_dim, vdim=2 * head_dim, scale=head_dim ** -0.5, diff=0.6)
+    left = dict(heads=heads, kv_heads=kv_heads, dim=head_dim, vdim=head_dim, scale=head_dim ** -0.5,
+                rot={"base": 500000.0, "dims": head_dim, "scaling": {"factor": 2.0}})
+    right = dict(heads=width // 128, kv_heads=width // 256, dim=128, vdim=128, conv=4)
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 16, "identity": 2, "top": 4}, "shared": {"ff": ff // 4}}
+    kinds = [("gla", gla, dense), ("gla", gla, moe), ("attention", diff, moe), ("parallel", {"left": left, "right": right}, moe)]
+    return {"architecture": "Muretar", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+            "layers": [dict(zip(("type", "mixer", "mlp"), kinds[i % 4])) for i in range(layers)]}
+
+
+def workload_muretar(args) -> int:
+    """Muretar beside a Llama of equal width, depth and vocabulary (see the module text)."""
+    import gc
+
+    import torch
+
+    layers = args.layers or 4
+    context = args.context
+    positions = max(context, PREFILL_TOKENS) + 64
+    sizes = {"1b": MODEL, "3b": MODEL_3B}
+    results = {}
+
+    def config(b):
+        return muretar_config(b["hidden_size"], b["num_attention_heads"], b["num_key_value_heads"], b["head_dim"],
+                              b["intermediate_size"], b["vocab_size"], layers)
+
+    if args.only:       # for profiles: the Muretar of the first size alone, a prompt or decode steps
+        runner, _cfg = make_runner(config(sizes["1b"]), layers, args.dtype, args.batch, max(args.batch * (context + 64), PREFILL_TOKENS + 64),
+                                   max_model_len=positions)
+        if args.only == "prefill":
+            sec = time_prefill(runner, PREFILL_TOKENS, max(1, args.steps // 8))
+            print(json.dumps({"only": "prefill", "model": "muretar_1b", "tokens": PREFILL_TOKENS, "ms": round(sec * 1e3, 3)}), flush=True)
+        else:
+            sec, _ = time_decode(runner, args.batch, args.steps, args.warmup, context, synthetic_cache=True)
+            print(json.dumps({"only": "decode", "model": "muretar_1b", "batch": args.batch, "ms_per_step": round(sec * 1e3, 4),
+                              "cache": "random numbers, no prompt was run"}), flush=True)
+        return 0
+    for name, base in sizes.items():
+        for what, raw in (("muretar", config(base)), ("llama", dict(base, tie_word_embeddings=False))):
+            runner, _cfg = make_runner(raw, layers, args.dtype, args.batch, max(args.batch * (context + 64), PREFILL_TOKENS + 64),
+                                       max_model_len=positions)
+            psec = time_prefill(runner, PREFILL_TOKENS, 3)
+            dsec, _ = time_decode(runner, args.batch, args.steps, args.warmup, context)
+            results[f"{what}_{name}"] = {"prefill_ms": round(psec * 1e3, 3), "prefill_tok_per_s": round(PREFILL_TOKENS / psec, 1),
+                                         "decode_ms_per_step": round(dsec * 1e3, 4), "decode_tok_per_s": round(args.batch / dsec, 1),
+                                         "graphs": len(runner._graphs)}
+            del runner
+            gc.collect()
+            torch.cuda.empty_cache()
+    first = results["muretar_1b"]
+    line = {
+        "metric": f"decode tok/s at batch {args.batch}, context {context} (Muretar at Llama 3.2 1B layer sizes, {layers} layers, random weights)",
+        "value": first["decode_tok_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": first["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
+        "config": {"model": "muretar-at-llama-sizes", "layers": layers, "global_batch": args.batch, "seq_len": context,
+                   "prefill_tokens": PREFILL_TOKENS, "experts": 16, "identity_experts": 2, "top": 4, "kv_block": BLOCK_SIZE,
+                   "parallelism": "single-gpu"},
+        "models": results,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -673,7 +751,7 @@ def main() -> int:
     ap.add_argument("--batch", default="8,1,64",
                     help="batch sizes of the decode steps: the first is the headline's, the others become points")
     ap.add_argument("--context", type=int, default=CONTEXT, help="context length that the decode steps end at")
-    ap.add_argument("--workload", choices=["decode1b", "long1b", "serve3b", "mixed8b", "dafidra", "rorevik", "dokanex"], default="decode1b")
+    ap.add_argument("--workload", choices=["decode1b", "long1b", "serve3b", "mixed8b", "dafidra", "rorevik", "dokanex", "muretar"], default="decode1b")
     ap.add_argument("--layers", type=int, default=None,
                     help="fewer layers than the model has, if memory or time needs it (both numbers are reported)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
@@ -711,6 +789,8 @@ def main() -> int:
         return workload_rorevik(args)
     if args.workload == "dokanex":
         return workload_dokanex(args)
+    if args.workload == "muretar":
+        return workload_muretar(args)
     args.layers = args.layers or MODEL["num_hidden_layers"]
     elem = 2 if args.dtype == "bf16" else 4
     big = args.batch if (args.no_points or args.only) else max(batches)

@@ -186,19 +186,97 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(TO* __restrict__ out, c
   for (int d = threadIdx.x; d < D; d += blockDim.x) out[m * D + d] = from_float<TO>((row[d] - mean) * rinv * w[d] + b[d]);
 }
 
+// The same for rows of whole 16-byte groups, at most VPT groups per thread: a thread keeps its values in registers
+// between the passes and every access is 16 bytes wide.  Few rows (decode steps) are a matter of latency: as many
+// threads per row as the row has groups.
+__device__ inline float sum4(const float4& v) { return (v.x + v.y) + (v.z + v.w); }
+__device__ inline float4 sub4(const float4& v, float m) { return make_float4(v.x - m, v.y - m, v.z - m, v.w - m); }
+__device__ inline float dot4(const float4& v) { return fmaf(v.w, v.w, fmaf(v.z, v.z, fmaf(v.y, v.y, v.x * v.x))); }
+__device__ inline float4 affine4(const float4& d, float r, const float4& w, const float4& b) {
+  return make_float4(fmaf(d.x * r, w.x, b.x), fmaf(d.y * r, w.y, b.y), fmaf(d.z * r, w.z, b.z), fmaf(d.w * r, w.w, b.w));
+}
+template <typename TO> __device__ inline void store4(TO* p, const float4& v);
+template <> __device__ inline void store4<float>(float* p, const float4& v) { *reinterpret_cast<float4*>(p) = v; }
+template <> __device__ inline void store4<bf16_t>(bf16_t* p, const float4& v) {
+  *reinterpret_cast<uint2*>(p) = make_uint2(f32x2_to_bf16x2_bits(v.x, v.y), f32x2_to_bf16x2_bits(v.z, v.w));
+}
+
+// mean and 1 / sqrt(variance + eps) of a row whose groups sit in v[VPT] (groups beyond the row are zero and not counted);
+// v becomes the deviations from the mean
+template <int VPT>
+__device__ inline float centre_and_scale(float4 (&v)[VPT], int groups, int D, float eps, float* scratch) {
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) s += sum4(v[i]);
+  const float mean = block_sum(s, scratch) / D;
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const bool in = (int)(threadIdx.x + i * blockDim.x) < groups;
+    v[i] = in ? sub4(v[i], mean) : make_float4(0.f, 0.f, 0.f, 0.f);
+    q += dot4(v[i]);
+  }
+  return 1.0f / sqrtf(block_sum(q, scratch) / D + eps);
+}
+
+template <typename TO, int VPT>
+__global__ __launch_bounds__(1024) void layer_norm_wide_kernel(TO* __restrict__ out, const float* __restrict__ x, const int* __restrict__ rows,
+                                                               const float* __restrict__ w, const float* __restrict__ b, float eps, int D,
+                                                               int x_rows) {
+  __shared__ float scratch[16];
+  const long m = blockIdx.x;
+  const long r = rows ? rows[m] : m;
+  const bool ok = r >= 0 && r < x_rows;
+  const int groups = D / 4;
+  float4 v[VPT], wv[VPT], bv[VPT];
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int g = threadIdx.x + i * blockDim.x;
+    const bool in = g < groups;
+    v[i] = !in ? make_float4(0.f, 0.f, 0.f, 0.f) : ok ? reinterpret_cast<const float4*>(x + r * D)[g] : make_float4(NAN, NAN, NAN, NAN);
+    wv[i] = in ? reinterpret_cast<const float4*>(w)[g] : make_float4(0.f, 0.f, 0.f, 0.f);
+    bv[i] = in ? reinterpret_cast<const float4*>(b)[g] : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  const float rinv = centre_and_scale<VPT>(v, groups, D, eps, scratch);
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int g = threadIdx.x + i * blockDim.x;
+    if (g < groups) store4<TO>(out + m * D + 4 * (long)g, affine4(v[i], rinv, wv[i], bv[i]));
+  }
+}
+
+// threads per row and groups per thread for the wide kernels: few rows, a thread per group (latency); many rows, fewer, fatter threads
+static inline bool wide_row_shape(int T, int D, int& threads, int& vpt) {
+  if (D % 4) return false;
+  const int groups = D / 4;
+  threads = T <= 512 ? groups : (groups + 3) / 4;
+  threads = threads > 1024 ? 1024 : ((threads + PI_WAVE - 1) / PI_WAVE) * PI_WAVE;
+  vpt = (groups + threads - 1) / threads;
+  return vpt <= 4;
+}
+
 extern "C" int pi_layer_norm(void* out, int out_dtype, const float* x, const int* rows, const float* w, const float* b, float eps,
                              int M, int D, int x_rows, hipStream_t stream) {
   PI_REQUIRE(M >= 0 && D > 0 && D <= 16000 && x_rows >= 0, "layer norm: bad sizes M=%d D=%d", M, D);
   PI_REQUIRE(out && x && w && b, "layer norm: output, input, weight and bias are needed");
+  PI_REQUIRE(out_dtype == PI_F32 || out_dtype == PI_BF16, "layer norm: unsupported dtype %d", out_dtype);
   if (M == 0) return 0;
+  int wide_threads = 0, vpt = 0;
+  const bool aligned = (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)b % 16 == 0 && (uintptr_t)out % 16 == 0;
+  if (aligned && wide_row_shape(M, D, wide_threads, vpt)) {
+#define LN_GO(TO, V) hipLaunchKernelGGL((layer_norm_wide_kernel<TO, V>), dim3(M), dim3(wide_threads), 0, stream, (TO*)out, x, rows, w, b, eps, D, x_rows)
+#define LN_PICK(TO) do { if (vpt <= 1) LN_GO(TO, 1); else if (vpt <= 2) LN_GO(TO, 2); else LN_GO(TO, 4); } while (0)
+    if (out_dtype == PI_F32) LN_PICK(float); else LN_PICK(bf16_t);
+#undef LN_PICK
+#undef LN_GO
+    return pi_check_launch("layer_norm_wide");
+  }
   const int threads = D >= 1024 ? 256 : (D >= 256 ? 128 : 64);
   const size_t lds = (size_t)D * sizeof(float);
   if (out_dtype == PI_F32)
     hipLaunchKernelGGL(layer_norm_kernel<float>, dim3(M), dim3(threads), lds, stream, (float*)out, x, rows, w, b, eps, D, x_rows);
-  else if (out_dtype == PI_BF16)
-    hipLaunchKernelGGL(layer_norm_kernel<bf16_t>, dim3(M), dim3(threads), lds, stream, (bf16_t*)out, x, rows, w, b, eps, D, x_rows);
   else
-    return pi_fail("layer norm: unsupported dtype %d", out_dtype);
+    hipLaunchKernelGGL(layer_norm_kernel<bf16_t>, dim3(M), dim3(threads), lds, stream, (bf16_t*)out, x, rows, w, b, eps, D, x_rows);
   return pi_check_launch("layer_norm");
 }
 
@@ -255,6 +333,73 @@ __global__ __launch_bounds__(256) void sandwich_norm_add_kernel(float* __restric
   for (int d = threadIdx.x; d < D; d += blockDim.x) h[t * D + d] = from_float<TH>((row[d] - mean) * rinv * nw[d] + nb[d]);
 }
 
+// The same with the row in registers and 16-byte accesses (see layer_norm_wide_kernel).
+template <typename TH, int VPT>
+__global__ __launch_bounds__(1024) void sandwich_norm_add_wide_kernel(float* __restrict__ x, TH* __restrict__ h, const float* __restrict__ a,
+                                                                      const float* __restrict__ a_bias, const float* __restrict__ wa,
+                                                                      const float* __restrict__ b, const float* __restrict__ wb,
+                                                                      const float* __restrict__ pw, const float* __restrict__ pb,
+                                                                      const float* __restrict__ nw, const float* __restrict__ nb,
+                                                                      float eps, int D) {
+  __shared__ float scratch[32];
+  const long t = blockIdx.x;
+  const int groups = D / 4;
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  float4 y[VPT], xo[VPT];
+  float sa = 0.f, sb = 0.f;
+  {
+    float4 vb[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int g = threadIdx.x + i * blockDim.x;
+      const bool in = g < groups;
+      y[i] = in ? reinterpret_cast<const float4*>(a + t * D)[g] : zero;
+      if (in && a_bias) {
+        const float4 ab = reinterpret_cast<const float4*>(a_bias)[g];
+        y[i] = make_float4(y[i].x + ab.x, y[i].y + ab.y, y[i].z + ab.z, y[i].w + ab.w);
+      }
+      vb[i] = (in && b) ? reinterpret_cast<const float4*>(b + t * D)[g] : zero;
+      xo[i] = in ? reinterpret_cast<const float4*>(x + t * D)[g] : zero;
+      sa += dot4(y[i]);
+      sb += dot4(vb[i]);
+    }
+    if (wa) {
+      block_sum2(sa, sb, scratch);
+      const float ra = 1.0f / sqrtf(sa / D + eps), rb = b ? 1.0f / sqrtf(sb / D + eps) : 0.f;
+#pragma unroll
+      for (int i = 0; i < VPT; ++i) {
+        const int g = threadIdx.x + i * blockDim.x;
+        if (g >= groups) continue;
+        const float4 w1 = reinterpret_cast<const float4*>(wa)[g];
+        float4 v = make_float4(y[i].x * ra * w1.x, y[i].y * ra * w1.y, y[i].z * ra * w1.z, y[i].w * ra * w1.w);
+        if (b) {
+          const float4 w2 = reinterpret_cast<const float4*>(wb)[g];
+          v = make_float4(0.5f * (v.x + vb[i].x * rb * w2.x), 0.5f * (v.y + vb[i].y * rb * w2.y), 0.5f * (v.z + vb[i].z * rb * w2.z),
+                          0.5f * (v.w + vb[i].w * rb * w2.w));
+        }
+        y[i] = v;
+      }
+    }
+  }
+  float rinv = centre_and_scale<VPT>(y, groups, D, eps, scratch);
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int g = threadIdx.x + i * blockDim.x;
+    if (g >= groups) continue;
+    const float4 l = affine4(y[i], rinv, reinterpret_cast<const float4*>(pw)[g], reinterpret_cast<const float4*>(pb)[g]);
+    xo[i] = make_float4(xo[i].x + l.x, xo[i].y + l.y, xo[i].z + l.z, xo[i].w + l.w);
+    reinterpret_cast<float4*>(x + t * D)[g] = xo[i];
+  }
+  if (!nw) return;
+  rinv = centre_and_scale<VPT>(xo, groups, D, eps, scratch);
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int g = threadIdx.x + i * blockDim.x;
+    if (g < groups)
+      store4<TH>(h + t * D + 4 * (long)g, affine4(xo[i], rinv, reinterpret_cast<const float4*>(nw)[g], reinterpret_cast<const float4*>(nb)[g]));
+  }
+}
+
 extern "C" int pi_sandwich_norm_add(float* x, void* h, int h_dtype, const float* a, const float* a_bias, const float* wa,
                                     const float* b, const float* wb, const float* pw, const float* pb, const float* nw,
                                     const float* nb, float eps, int T, int D, hipStream_t stream) {
@@ -262,47 +407,66 @@ extern "C" int pi_sandwich_norm_add(float* x, void* h, int h_dtype, const float*
   PI_REQUIRE(x && a && pw && pb, "norm and add: the stream, a result and the norm's weight and bias are needed");
   PI_REQUIRE(!b || (wa && wb), "norm and add: two branches need both their weights");
   PI_REQUIRE(!nw || (nb && h), "norm and add: the next norm needs its bias and a place for its result");
+  PI_REQUIRE(!nw || h_dtype == PI_F32 || h_dtype == PI_BF16, "norm and add: unsupported activation dtype %d", h_dtype);
   if (T == 0) return 0;
+  const bool f32 = !nw || h_dtype == PI_F32;
+  int wide_threads = 0, vpt = 0;
+  bool aligned = true;
+  for (const void* p : {(const void*)x, (const void*)h, (const void*)a, (const void*)a_bias, (const void*)wa, (const void*)b, (const void*)wb,
+                        (const void*)pw, (const void*)pb, (const void*)nw, (const void*)nb})
+    aligned = aligned && (uintptr_t)p % 16 == 0;
+  if (aligned && wide_row_shape(T, D, wide_threads, vpt)) {
+#define SW_GO(TH, V) hipLaunchKernelGGL((sandwich_norm_add_wide_kernel<TH, V>), dim3(T), dim3(wide_threads), 0, stream, x, (TH*)h, a, a_bias, wa, b, wb, pw, pb, nw, nb, eps, D)
+#define SW_PICK(TH) do { if (vpt <= 1) SW_GO(TH, 1); else if (vpt <= 2) SW_GO(TH, 2); else SW_GO(TH, 4); } while (0)
+    if (f32) SW_PICK(float); else SW_PICK(bf16_t);
+#undef SW_PICK
+#undef SW_GO
+    return pi_check_launch("sandwich_norm_add_wide");
+  }
   const int threads = D >= 1024 ? 256 : (D >= 256 ? 128 : 64);
   const size_t lds = (size_t)D * sizeof(float);
-  if (!nw || h_dtype == PI_F32)
+  if (f32)
     hipLaunchKernelGGL(sandwich_norm_add_kernel<float>, dim3(T), dim3(threads), lds, stream, x, (float*)h, a, a_bias, wa, b, wb, pw, pb, nw, nb, eps, D);
-  else if (h_dtype == PI_BF16)
-    hipLaunchKernelGGL(sandwich_norm_add_kernel<bf16_t>, dim3(T), dim3(threads), lds, stream, x, (bf16_t*)h, a, a_bias, wa, b, wb, pw, pb, nw, nb, eps, D);
   else
-    return pi_fail("norm and add: unsupported activation dtype %d", h_dtype);
+    hipLaunchKernelGGL(sandwich_norm_add_kernel<bf16_t>, dim3(T), dim3(threads), lds, stream, x, (bf16_t*)h, a, a_bias, wa, b, wb, pw, pb, nw, nb, eps, D);
   return pi_check_launch("sandwich_norm_add");
 }
 
 // ---------------------------------------------------------------- two attention maps into one head
 // Differential attention: head n of kv group g holds the results a1 and a2 of two softmax maps over the same
-// values.  In `attn` the maps are heads of their own, ordered [g][map][head within group] (so that the
-// attention kernels see map m of group g as kv head 2 g + m).  out[t, n, :] = mult * o / sqrt(mean(o^2) + eps),
+// values.  In `attn` the maps are heads of their own, and a head's value vector may come in `split` equal pieces
+// (each attended as a head of its own, so that heads whose values are a multiple of their keys' width fit kernels
+// that want both alike): heads are ordered [g][map][piece][head within group], so that piece p of map m of group g
+// is kv head (2 g + m) * split + p of the attention.  out[t, n, :] = mult * o / sqrt(mean(o^2) + eps),
 // o = a1 - lam * a2, float32; one wave per (token, head).
 template <typename TO, typename TI>
 __global__ __launch_bounds__(PI_WAVE) void diff_combine_kernel(TO* __restrict__ out, const TI* __restrict__ attn, float lam, float eps,
-                                                               float mult, int H, int G, int dv) {
+                                                               float mult, int H, int G, int dv, int split) {
   const long t = blockIdx.x;
   const int n = blockIdx.y, lane = threadIdx.x;
-  const int per = H / G, g = n / per, i = n % per;
-  const TI* a1 = attn + (t * 2 * H + (long)(2 * g) * per + i) * dv;
-  const TI* a2 = a1 + (long)per * dv;
+  const int per = H / G, g = n / per, i = n % per, w = dv / split;      // w: a piece's width
+  const TI* row = attn + t * 2 * H * dv;
+  const long map_step = (long)split * per * w;                          // from map 1 to map 2 of a group
   float ss = 0.f;
   for (int c = lane; c < dv; c += PI_WAVE) {
-    const float o = fmaf(-lam, to_float(a2[c]), to_float(a1[c]));
+    const long at = (((long)(2 * g) * split + c / w) * per + i) * w + c % w;
+    const float o = fmaf(-lam, to_float(row[at + map_step]), to_float(row[at]));
     ss = fmaf(o, o, ss);
   }
   const float r = mult / sqrtf(wave_sum(ss) / dv + eps);
-  for (int c = lane; c < dv; c += PI_WAVE)
-    out[(t * H + n) * dv + c] = from_float<TO>(fmaf(-lam, to_float(a2[c]), to_float(a1[c])) * r);
+  for (int c = lane; c < dv; c += PI_WAVE) {
+    const long at = (((long)(2 * g) * split + c / w) * per + i) * w + c % w;
+    out[(t * H + n) * dv + c] = from_float<TO>(fmaf(-lam, to_float(row[at + map_step]), to_float(row[at])) * r);
+  }
 }
 
 extern "C" int pi_diff_combine(void* out, int out_dtype, const void* attn, int in_dtype, float lam, float eps, float mult, int T, int H,
-                               int G, int dv, hipStream_t stream) {
+                               int G, int dv, int split, hipStream_t stream) {
   PI_REQUIRE(T >= 0 && H > 0 && H <= 65535 && G > 0 && H % G == 0 && dv > 0, "two maps: bad sizes heads=%d kv_heads=%d vdim=%d", H, G, dv);
+  PI_REQUIRE(split >= 1 && dv % split == 0, "two maps: values of %d do not come in %d equal pieces", dv, split);
   if (T == 0) return 0;
   const dim3 grid(T, H), block(PI_WAVE);
-#define DC_GO(TO, TI) hipLaunchKernelGGL((diff_combine_kernel<TO, TI>), grid, block, 0, stream, (TO*)out, (const TI*)attn, lam, eps, mult, H, G, dv)
+#define DC_GO(TO, TI) hipLaunchKernelGGL((diff_combine_kernel<TO, TI>), grid, block, 0, stream, (TO*)out, (const TI*)attn, lam, eps, mult, H, G, dv, split)
   if (out_dtype == PI_F32 && in_dtype == PI_F32) DC_GO(float, float);
   else if (out_dtype == PI_BF16 && in_dtype == PI_BF16) DC_GO(bf16_t, bf16_t);
   else if (out_dtype == PI_BF16 && in_dtype == PI_F32) DC_GO(bf16_t, float);

@@ -604,16 +604,17 @@ def sandwich_norm_add(x: torch.Tensor, a: torch.Tensor, post, eps: float, nxt=No
 
 
 def diff_combine(out: torch.Tensor, attn: torch.Tensor, lam: float, eps: float, mult: float, heads: int, kv_heads: int,
-                 value_dim: int) -> None:
+                 value_dim: int, split: int = 1) -> None:
     """Two attention maps per head into one result: ``attn`` [T, 2 * heads * value_dim] holds the maps as heads of
-    their own in the order [kv group][map][head within the group]; out[t, n, :] = mult * o / sqrt(mean(o^2) + eps) with
+    their own, a head's values in ``split`` equal pieces that were attended as heads of their own, in the order
+    [kv group][map][piece][head within the group]; out[t, n, :] = mult * o / sqrt(mean(o^2) + eps) with
     o = map 1 - lam * map 2 of head n, float32 arithmetic."""
     _gpu(out, attn)
     T = out.shape[0]
     if tuple(out.shape) != (T, heads * value_dim) or tuple(attn.shape) != (T, 2 * heads * value_dim) or not (out.is_contiguous() and attn.is_contiguous()):
         raise KernelError(f"two maps: expected contiguous [{T}, {2 * heads * value_dim}] -> [{T}, {heads * value_dim}], got {tuple(attn.shape)} -> {tuple(out.shape)}")
     _lib.call("core", "pi_diff_combine", out.data_ptr(), _dt(out), attn.data_ptr(), _dt(attn), float(lam), float(eps), float(mult), T,
-              int(heads), int(kv_heads), int(value_dim), _stream())
+              int(heads), int(kv_heads), int(value_dim), int(split), _stream())
 
 
 EPI_RELU2 = 5        # the matrix-core products' epilogue: max(c, 0)^2 rounded to bfloat16

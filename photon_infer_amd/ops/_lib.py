@@ -43,7 +43,7 @@ _SIGNATURES = {
         "pi_relu_squared": [P, I, P, L, P],
         "pi_layer_norm": [P, I, P, P, P, P, F, I, I, I, P],
         "pi_sandwich_norm_add": [P, P, I, P, P, P, P, P, P, P, P, P, F, I, I, P],
-        "pi_diff_combine": [P, I, P, I, F, F, F, I, I, I, I, P],
+        "pi_diff_combine": [P, I, P, I, F, F, F, I, I, I, I, I, P],
         "pi_paged_attention_general_ranges": [I, I, I],
         "pi_rope_table": [P, P, P, I, I, F, P],
         "pi_sample": [P, P, L, P, P, I, I, P, L, P],

@@ -164,9 +164,11 @@ def run_paged_part(part, h, want, cuts_list, tdt, page, tol, what, D):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("sizes", [(4, 2, 16, 24), (4, 1, 64, 64), (6, 3, 12, 10), (1, 1, 48, 48), (2, 2, 32, 64), (8, 2, 128, 128)])
+@pytest.mark.parametrize("sizes", [(4, 2, 16, 24), (4, 1, 64, 64), (6, 3, 12, 10), (1, 1, 48, 48), (2, 2, 32, 64), (8, 2, 128, 128), (2, 1, 16, 48),
+                                   (4, 2, 64, 128)])
 def test_differential_attention_whole_in_portions_and_token_by_token(dtype, sizes):
-    """One token far back is loud; the second map's vectors make a lambda far from ``diff``."""
+    """One token far back is loud; the second map's vectors make a lambda far from ``diff``.  Values two and three times as
+    wide as keys are attended in pieces by the bfloat16 engine."""
     H, G, d, dv = sizes
     D, T, page, eps, scale, diff = 72, 150, 16, 1e-5, 0.11, 0.35
     tdt = TORCH[dtype]
@@ -183,6 +185,7 @@ def test_differential_attention_whole_in_portions_and_token_by_token(dtype, size
     part = make_part("differential_attention", W, tdt, hidden_size=D, num_heads=H, num_kv_heads=G, head_dim=d, value_dim=dv, scale=scale, diff=diff,
                      eps=eps, accumulate=False)
     assert abs(part.lam - lam) < 1e-12
+    assert part.split == (dv // d if dtype == "bfloat16" and d % 16 == 0 and dv % d == 0 else 1)
     run_paged_part(part, h, want, ([T], [64, 7, 2, 77], [T - 12] + [1] * 12), tdt, page, 1e-4 if dtype == "float32" else 5e-2, f"{sizes}", D)
 
 
