@@ -485,7 +485,8 @@ __global__ __launch_bounds__(256) void rope_kv_write_wide_kernel(
     long v_stride, const int* __restrict__ positions, const int* __restrict__ req_of_token, const float* __restrict__ table,
     int rotate, int T, int nh, int nkv_write, int nkv, int hd, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_table, int table_width, int page_size, long num_pages, long rot_items,
-    const float* __restrict__ part, int splits, long part_stride, int ncols, int q_col, int k_col, int v_col) {
+    const float* __restrict__ part, int splits, long part_stride, int ncols, int q_col, int k_col, int v_col,
+    const float* __restrict__ bias) {
   const long idx = (long)blockIdx.x * 256 + threadIdx.x;
   const int units = hd / 16, heads = nh + nkv_write;
   if (idx < rot_items) {
@@ -508,7 +509,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_wide_kernel(
       dst = k_cache + ((page * nkv + g) * page_size + (pos % page_size)) * hd;
       col = k_col + g * hd;
     }
-    if (!part && !rotate && dst == src) return;
+    if (!part && !rotate && !bias && dst == src) return;
     typedef float quad_t __attribute__((ext_vector_type(4)));
     float a[8], b[8];                            // the features and their partners, float32
     if (part) {
@@ -541,6 +542,16 @@ __global__ __launch_bounds__(256) void rope_kv_write_wide_kernel(
         b[2 * w] = __uint_as_float(hw[w] << 16); b[2 * w + 1] = __uint_as_float(hw[w] & 0xffff0000u);
       }
     }
+    if (bias) {                                  // the projection's bias, by column, before the rotation
+      const float* bp = bias + col + d;
+      const quad_t a0 = *reinterpret_cast<const quad_t*>(bp), a1 = *reinterpret_cast<const quad_t*>(bp + 4);
+      const quad_t b0 = *reinterpret_cast<const quad_t*>(bp + hd / 2), b1 = *reinterpret_cast<const quad_t*>(bp + hd / 2 + 4);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        a[e] += e < 4 ? a0[e] : a1[e - 4];
+        b[e] += e < 4 ? b0[e] : b1[e - 4];
+      }
+    }
     if (rotate) {
       const float* c = table + t * hd + d;
       const float* sn = c + hd / 2;
@@ -571,8 +582,10 @@ __global__ __launch_bounds__(256) void rope_kv_write_wide_kernel(
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const long t = t0 + (i < n ? i : 0);
-    if (part) {
-      const bf16_t r = from_float<bf16_t>(split_sum(part, splits, part_stride, t * ncols + v_col + g * hd + d));
+    if (part || bias) {
+      float f = part ? split_sum(part, splits, part_stride, t * ncols + v_col + g * hd + d) : to_float(v[t * v_stride + (long)g * hd + d]);
+      if (bias) f += bias[v_col + g * hd + d];
+      const bf16_t r = from_float<bf16_t>(f);
       val[i] = *reinterpret_cast<const uint16_t*>(&r);
     } else {
       val[i] = *reinterpret_cast<const uint16_t*>(v + t * v_stride + (long)g * hd + d);
@@ -627,7 +640,7 @@ extern "C" int pi_rope_kv_write(void* q, long q_stride, const void* k, long k_st
                               : (!write_kv || (k_stride % 8 == 0 && ((uintptr_t)k % 16 == 0)));
   const bool aligned = hd % 16 == 0 && q_stride % 8 == 0 && ((uintptr_t)q % 16 == 0) && (!table || (uintptr_t)table % 16 == 0) &&
                        source_ok && (!write_kv || (((uintptr_t)k_cache % 16 == 0) && ((uintptr_t)v_cache % 8 == 0) && page_size % 4 == 0));
-  if (dtype == PI_BF16 && usual && aligned && T >= 16 && vd == hd && !bias) {
+  if (dtype == PI_BF16 && usual && aligned && T >= 16 && vd == hd && (!bias || ((uintptr_t)bias % 16 == 0 && q_col % 4 == 0 && k_col % 4 == 0))) {
     const int nkv_w = write_kv ? nkv : 0;
     const long rot_items = (long)T * (nh + nkv_w) * (hd / 16);
     const long v_items = write_kv ? (long)((T + 3) / 4) * nkv * hd : 0;
@@ -636,7 +649,7 @@ extern "C" int pi_rope_kv_write(void* q, long q_stride, const void* k, long k_st
     hipLaunchKernelGGL(rope_kv_write_wide_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (bf16_t*)q, q_stride,
                        (const bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, positions, req_of_token, table,
                        rotary_dim > 0 ? 1 : 0, T, nh, nkv_w, nkv, hd, (bf16_t*)k_cache, (bf16_t*)v_cache, block_table,
-                       table_width, page_size, num_pages, rot_items, part, splits, (long)T * ncols, ncols, q_col, k_col, v_col);
+                       table_width, page_size, num_pages, rot_items, part, splits, (long)T * ncols, ncols, q_col, k_col, v_col, bias);
     return pi_check_launch("rope_kv_write_wide");
   }
   PI_REQUIRE(heads <= 65535, "rope_kv_write: too many heads (%d)", heads);
