@@ -40,7 +40,7 @@ def state_ctx(q_lens, slots):
     """The fields of a StepContext that the kernels of mixers with a state read."""
     q_start = np.zeros(len(q_lens) + 1, np.int32)
     np.cumsum(q_lens, out=q_start[1:])
-    return SimpleNamespace(T=int(sum(q_lens)), R=len(q_lens), max_q_len=max(q_lens),
+    return SimpleNamespace(T=int(sum(q_lens)), R=len(q_lens), max_q_len=max(q_lens), q_lens=list(q_lens),
                            q_start=torch.from_numpy(q_start).to(DEV), slots=torch.tensor(slots, dtype=torch.int32, device=DEV))
 
 
@@ -318,6 +318,28 @@ def test_gated_linear_attention_walk_whole_in_portions_and_token_by_token(sizes)
         for n in T:
             close(got[n], want[n].reshape(T[n], -1), f"{sizes} {n} cut {cuts[n]}", 5e-5)
         assert bool((state[1] == 0).all()) and bool((state[3] == 0).all())
+
+
+@pytest.mark.parametrize("sizes", [(2, 24, 16, 8.0), (3, 20, 28, 3.5), (2, 128, 64, 2.0), (1, 40, 200, 1.0)])
+def test_long_portions_of_the_linear_walk_beside_short_ones(sizes):
+    """Portions of hundreds of tokens (many chunks of the walk) beside single tokens and a short portion; the state a portion
+    leaves is the one the next step starts from, whatever the cutting."""
+    from photon_infer_amd import ops
+    H, d, dv, tau = sizes
+    T = {"a": 700, "b": 300, "c": 9}
+    consts = {"a_bias": randn(H * d, seed=2), "tau": tau}
+    data, want = {}, {}
+    for i, (n, t) in enumerate(T.items()):
+        q, k, v, z = randn(t, H, d, seed=10 + i), randn(t, H, d, seed=20 + i), randn(t, H, dv, seed=30 + i), randn(t, H, d, seed=40 + i, scale=2.0) + 3.0
+        data[n] = (torch.cat([q.reshape(t, -1), k.reshape(t, -1), v.reshape(t, -1)], dim=1), z.reshape(t, -1))
+        alpha = P.sigmoid(z + consts["a_bias"].view(H, d)) ** (1.0 / tau)
+        want[n] = torch.stack([P.decayed_outer_walk(q[:, h] * d ** -0.5, k[:, h], v[:, h], alpha[:, h]) for h in range(H)], 1)
+    slot = {"a": 0, "b": 2, "c": 3}
+    for cuts in ({"a": [700], "b": [300], "c": [9]}, {"a": [256, 1, 300, 143], "b": [1, 299], "c": [1]}, {"a": [129, 571], "b": [44, 256], "c": [3]}):
+        got, state = walk("decayed_outer", data, T, slot, cuts, (H, H, d, dv), consts)
+        for n in T:
+            close(got[n], want[n].reshape(T[n], -1), f"{sizes} {n} cut {cuts[n]}", 1e-4)
+        assert bool((state[1] == 0).all())
 
 
 @pytest.mark.parametrize("decode", [False, True])
@@ -634,6 +656,17 @@ def test_mixed_batches_with_pages_and_slots_used_again(name, dtype, model_dirs, 
     assert runner.cache.max_slots == 4
     run_checked(runner, steps, str(tmp_path), model_dirs[name], reqs, dtype, "mixed")
     assert all(g.pool.num_allocated == 0 for g in runner.cache.groups)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_long_prompt_whole_and_in_two_long_portions(dtype, model_dirs, tmp_path):
+    """600 tokens whole, and in two long portions and a single token."""
+    vocab = TM.ALL["A"][0]["vocab"]
+    reqs = {"w": random_tokens(600, vocab, 11), "p": random_tokens(600, vocab, 11)}
+    steps = cut_steps("w", reqs["w"], [600])
+    steps += cut_steps("p", reqs["p"], [301, 298, 1], first_step=len(steps))
+    runner = runner_for(model_dirs["A"], "A", dtype, live_token_need(steps))
+    run_checked(runner, steps, str(tmp_path), model_dirs["A"], reqs, dtype, "long prompt")
 
 
 @pytest.mark.parametrize("name", ["A", "C"])
