@@ -112,8 +112,7 @@ class GatedDeltaRule(Mixer):
     * q, k, v as above (convolutions, silu, unit vectors, q times ``key_dim^-1/2``);
     * ``beta = sigmoid(W_b h)`` and ``decay = exp(-exp(A_log_n) softplus(W_a h + dt_bias_n))``, one each per head;
     * per head: ``S <- decay S``, ``u = beta (v - S^T k)``, ``S <- S + k u^T``, ``o = S^T q``;
-    * each head's o RMS-normalised over value_dim with the weight ``norm`` (shared by the heads), times
-      ``silu(W_g h)``, then ``W_o``.
+    * ``y = W_o (silu(W_g h) * concat_n(rms(o_n) * norm))`` with one norm weight of ``value_dim`` for all heads.
 
     One projection gives everything that is read from h, as float32: rows [q | k | v | b | a | g]."""
 

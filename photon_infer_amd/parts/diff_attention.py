@@ -4,8 +4,9 @@ difference (Ye et al., "Differential Transformer").
 With input h, ``heads`` query heads and ``kv_heads`` key / value heads (query head n reads key / value
 head ``n // (heads / kv_heads)``), keys of ``head_dim`` and values of ``value_dim``:
 
-* ``q = W_q h + b_q`` has ``heads * 2 * head_dim`` rows and ``k = W_k h + b_k`` has ``kv_heads * 2 * head_dim`` rows, laid
-  out head by head as [map 1 | map 2]; ``v = W_v h + b_v`` (``kv_heads * value_dim``).  No rotation.
+* ``q = W_q h + b_q`` (``heads * 2 * head_dim`` rows) and ``k = W_k h + b_k`` (``kv_heads * 2 * head_dim`` rows): a head's
+  rows are map 1's, then map 2's; ``v = W_v h + b_v`` (``kv_heads * value_dim`` rows) serves both maps.  Positions enter
+  through the causal mask alone.
 * per head and map m: ``a_m = softmax(scale * q_m K_m^T) V`` over the keys at positions <= the query's;
 * ``lam = exp(<lq1, lk1>) - exp(<lq2, lk2>) + diff`` (one number per layer, from four vectors of ``head_dim``);
 * ``o = a_1 - lam * a_2``, divided by the root mean square of its ``value_dim`` entries (eps inside the root, no

@@ -6,8 +6,8 @@ With input h, ``heads`` heads with keys of ``key_dim`` and values of ``value_dim
 * ``q = W_q h * key_dim^-1/2``, ``k = W_k h``, ``v = W_v h`` (no biases);
 * a decay per head and key channel, ``alpha = sigmoid(W_a2 (W_a1 h) + b_a2)^(1 / tau)`` (a low-rank projection);
 * per head, state S [key_dim, value_dim]: ``S <- diag(alpha) S + k v^T``, ``o = S^T q``;
-* each head's o is RMS-normalised over value_dim with the weight ``norm`` (shared by the heads), heads concatenated,
-  times ``silu(W_g h)``, then ``W_o``.
+* ``y = W_o (silu(W_g h) * concat_n(rms(o_n) * norm))``: one norm weight of ``value_dim`` for all heads, the gate over
+  all heads' values at once.
 
 Decays, the state and the norm are float32 in both compute modes; q, k and v enter the recurrence as the float32
 results of their projection.  A request's state row holds S, is cleared when the request is admitted and carried from

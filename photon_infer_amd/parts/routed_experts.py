@@ -9,9 +9,9 @@ biases (``activation`` "silu"), or ``Wdown max(Wup h, 0)^2`` (``activation`` "re
 the weighted sum of the chosen experts' outputs (float32).
 
 Further options, each a constructor parameter: ``correction`` (a tensor of one number per router output that is
-added to the scores for the choice only; the weights stay the scores), ``identity`` (the last so many router outputs
-are identity experts: they have no tensors and their output is the input itself, times the weight), and ``shared``
-((prefix, feed-forward): an expert that runs for every token and is added).
+added to the scores for the choice only; the weights stay the scores), ``identity`` (so many identity experts, which take
+the last places among the router's outputs, own no matrices and contribute ``weight * h``), and ``shared``
+((prefix, feed-forward): one more feed-forward that every token goes through, added to the routed sum).
 
 The step's (token, choice) entries are sorted by expert on the device and each expert's rows go
 through grouped products; nothing is counted on the host.

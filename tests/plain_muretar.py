@@ -20,7 +20,7 @@ LN is a layer norm with weight and bias.  A layer's mixer is one of
 A feed-forward is dense and gated (silu), or routed: a softmax router over real and identity
 experts, a correction added for the choice only, the chosen scores divided by their sum, experts
 ``W_down relu(W_up h)^2``, identity experts that hand the input through, and a shared expert.
-A layer with ``weights_of: j`` runs layer j's tensors with a memory of its own.
+``weights_of: j`` in a layer's entry: the layer is run with the tensors named ``l<j>.`` and keeps its own cache or state.
 """
 from __future__ import annotations
 
