@@ -623,7 +623,7 @@ extern "C" int pi_rope_kv_write(void* q, long q_stride, const void* k, long k_st
                                 int k_col, int v_col, int vd, const float* bias, hipStream_t stream) {
   // bias: float32, one per column of the projection [q heads | k heads | v heads], found at q_col / k_col / v_col
   if (vd <= 0) vd = hd;
-  PI_REQUIRE(vd <= 256, "rope_kv_write: value width %d must be at most 256", vd);
+  PI_REQUIRE(vd <= 640, "rope_kv_write: value width %d must be at most 640", vd);      // as wide as the general attention kernel reads them
   PI_REQUIRE(T >= 0 && nh >= 0 && nkv >= 0 && hd > 0 && hd <= 256, "rope_kv_write: bad sizes T=%d heads=%d kv_heads=%d head_dim=%d", T, nh, nkv, hd);
   PI_REQUIRE(rotary_dim >= 0 && rotary_dim <= hd && rotary_dim % 2 == 0, "rope_kv_write: rotary_dim %d must be even and <= head_dim %d", rotary_dim, hd);
   PI_REQUIRE(rotary_dim == 0 || table != nullptr, "rope_kv_write: rotation asked for without a cos / sin table");

@@ -165,7 +165,7 @@ def run_paged_part(part, h, want, cuts_list, tdt, page, tol, what, D):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("sizes", [(4, 2, 16, 24), (4, 1, 64, 64), (6, 3, 12, 10), (1, 1, 48, 48), (2, 2, 32, 64), (8, 2, 128, 128), (2, 1, 16, 48),
-                                   (4, 2, 64, 128)])
+                                   (4, 2, 64, 128), (2, 1, 128, 384)])
 def test_differential_attention_whole_in_portions_and_token_by_token(dtype, sizes):
     """One token far back is loud; the second map's vectors make a lambda far from ``diff``.  Values two and three times as
     wide as keys are attended in pieces by the bfloat16 engine."""
